@@ -20,15 +20,29 @@ class NormSpec:
 
 
 @dataclass(frozen=True)
+class FrequencyScaling:
+    """Long wavelengths of a rotation are stretched: with l = 2 pi / f, a frequency stays where
+    l < original / high, becomes f / factor where l > original / low, and in between the blend
+    (1 - s) f / factor + s f with s = (original / l - low) / (high - low)."""
+    factor: float
+    low: float
+    high: float
+    original: float
+
+
+@dataclass(frozen=True)
 class PositionSpec:
     """Position encoding of a mixer.  kind "rope": rotate-half pairs (i, i+dim/2)
     with angle = position / theta^(2i/dim), from a table of `max_positions` rows; kind
     "rope_pairs": neighbouring pairs (2i, 2i+1) with the same angles, worked out by the kernels
-    from the frequencies theta^(-2i/dim), so no position is too far; kind "none": no encoding."""
+    from the frequencies theta^(-2i/dim), so no position is too far; kind "rope_half": the pairs
+    of "rope" with the angles worked out by the kernels as for "rope_pairs", the frequencies
+    optionally rescaled (`scaling`); kind "none": no encoding."""
     kind: str = "rope"
     theta: float = 10000.0
     dim: int = 0
     max_positions: int = 0
+    scaling: Optional[FrequencyScaling] = None      # kind "rope_half" only
 
 
 @dataclass(frozen=True)
@@ -68,6 +82,15 @@ class AttentionSpec:
     # the output projection's bias: None: taken when the checkpoint holds it, True: it must
     # hold it, False: it must not
     o_bias: Optional[bool] = None
+    # values shared across layers of a step: "source": this layer's values (before anything is
+    # mixed into them) are kept for the step's later layers; "mix": what this layer caches and
+    # attends to is (1 - lambda) v + lambda v_source, v_source the source layer's values of the
+    # same token and lambda a learned number; "off": the layer's values are its own, but its
+    # checkpoint may hold the (unused) number; None: no such thing
+    value_mix: Optional[str] = None
+    # the concatenated heads are multiplied, element by element, by sigmoid(W_g x), x the
+    # mixer's input, before the output projection
+    output_gate: bool = False
 
     @property
     def q_width(self) -> int:
@@ -95,10 +118,44 @@ class GatedMLPSpec:
     """down(act(gate(x)) * up(x))."""
     kind: str = "gated_mlp"
     intermediate_size: int = 0
-    activation: str = "silu"      # of the gate: "silu" or "gelu_tanh"
+    # of the gate: "silu" or "gelu_tanh"; or "clamped_swish": with g = min(gate x, limit) and
+    # u = clamp(up x, -limit, limit) the product is g sigmoid(alpha g) (u + 1)
+    activation: str = "silu"
     # biases of the three projections: None: taken when the checkpoint holds them, True: it
     # must hold them, False: it must not
     bias: Optional[bool] = None
+    limit: float = 0.0            # "clamped_swish" only
+    alpha: float = 1.0            # "clamped_swish" only
+
+
+@dataclass(frozen=True)
+class RoutedMLPSpec:
+    """Mixture of experts: a router chooses `top` of `n_experts` gated feed-forwards
+    down(silu(gate x) * up x) for every token, by the largest float32 logits W_router x, and
+    adds their outputs weighted by the softmax over the chosen logits alone."""
+    kind: str = "routed_mlp"
+    n_experts: int = 0
+    top: int = 0
+    intermediate_size: int = 0    # of one expert
+
+
+@dataclass(frozen=True)
+class StateSpaceSpec:
+    """Selective state-space mixer with one decay per head (Mamba-2): a recurrent mixer whose
+    state is one [state, head_dim] matrix per head, fed through a short causal convolution.
+    See `parts.ssm`."""
+    kind: str = "mamba2"
+    n_heads: int = 0
+    head_dim: int = 0             # columns of a head's state (its share of the inner width)
+    state: int = 0                # rows of a head's state: the size of B and C
+    groups: int = 1               # pairs of B and C, each shared by n_heads / groups heads
+    conv_taps: int = 4
+    norm_parts: int = 1           # the gated read-out is RMS-normed in this many equal parts
+    norm_eps: float = 1e-6
+
+    @property
+    def inner(self) -> int:
+        return self.n_heads * self.head_dim
 
 
 @dataclass(frozen=True)
@@ -230,6 +287,9 @@ class ModelSpec:
     eos_token_id: Optional[int]
     embedding_scale: float = 1.0         # the embedding rows are multiplied by this
     loop: Optional[LoopSpec] = None      # the schedule then has to be `looped_schedule`'s
+    embedding_norm: Optional[NormSpec] = None    # a norm on the embedding rows (None: none)
+    logit_scale: float = 1.0             # the head's products are multiplied by this,
+    logit_softcap: Optional[float] = None    # and then capped: c tanh(logit / c) (None: no cap)
 
     def validate(self) -> None:
         if not self.layers or not self.schedule:

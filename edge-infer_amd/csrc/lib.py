@@ -29,7 +29,11 @@ _SIGNATURES = {
         "ei_add_rmsnorm": [c_void_p, c_void_p, c_int, c_int, c_longlong, c_void_p, c_void_p,
                            c_float, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
         "ei_swiglu": [c_void_p, c_int, c_int, c_longlong, c_void_p, c_int, c_int, c_int, c_int,
-                      c_int, c_void_p, c_void_p],
+                      c_int, c_void_p, c_float, c_float, c_void_p],
+        "ei_norm_rows": [c_void_p, c_void_p, c_float, c_longlong, c_int, c_void_p],
+        "ei_gate_rows": [c_void_p, c_int, c_int, c_longlong, c_longlong, c_int, c_void_p, c_int,
+                         c_longlong, c_int, c_void_p],
+        "ei_scale_cap": [c_void_p, c_float, c_float, c_longlong, c_void_p],
         "ei_norm_add_norm": [c_void_p, c_void_p, c_int, c_int, c_longlong, c_void_p, c_void_p,
                              c_float, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p],
         "ei_concat_cast": [c_void_p, c_void_p, c_void_p, c_int, c_longlong, c_int, c_void_p],
@@ -48,10 +52,32 @@ _SIGNATURES = {
                                   c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                   c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                   c_void_p],
+        "ei_head_store": [c_void_p, c_int, c_int, c_longlong, c_longlong, c_void_p, c_void_p,
+                          c_float, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
+                          c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int,
+                          c_int, c_int, c_int, c_int, c_void_p],
         "ei_projection_norm_store": [c_void_p, c_int, c_int, c_longlong, c_void_p, c_void_p, c_void_p,
                                      c_float, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                      c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                      c_int, c_void_p],
+    },
+    "ssm": {
+        "ei_ssm_state_floats": [c_int, c_int, c_int, c_int, c_int],
+        "ei_ssm_conv": [c_void_p, c_int, c_int, c_longlong, c_longlong, c_void_p, c_void_p,
+                        c_void_p, c_longlong, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                        c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                        c_int, c_void_p],
+        "ei_ssm_scan": [c_void_p, c_void_p, c_int, c_int, c_longlong, c_longlong, c_void_p,
+                        c_void_p, c_void_p, c_void_p, c_longlong, c_void_p, c_void_p, c_void_p,
+                        c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+        "ei_ssm_out": [c_void_p, c_void_p, c_int, c_int, c_longlong, c_longlong, c_void_p,
+                       c_float, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+    },
+    "moe": {
+        "ei_moe_route": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                         c_int, c_int, c_void_p],
+        "ei_moe_experts": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
+                           c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     },
     "delta_rule": {
         "ei_delta_conv": [c_void_p, c_int, c_int, c_longlong, c_int, c_void_p, c_int, c_void_p,
@@ -302,15 +328,17 @@ def add_rmsnorm(residual: torch.Tensor, delta: Optional[torch.Tensor], weight: t
     _check(lib, status, "add_rmsnorm")
 
 
-GATE_ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
+GATE_ACTIVATIONS = {"silu": 0, "gelu_tanh": 1, "clamped_swish": 2}
 
 
 def swiglu(gate_up: torch.Tensor, out: torch.Tensor, strip: int = 0,
-           activation: str = "silu", bias: Optional[torch.Tensor] = None) -> None:
+           activation: str = "silu", bias: Optional[torch.Tensor] = None,
+           limit: float = 0.0, alpha: float = 1.0) -> None:
     """out = act(gate) * up of [n, 2*inter] rows (or float32 slices of them), act "silu" or
-    "gelu_tanh".  strip = 0: the gate columns come first, then the up columns; strip > 0:
-    `strip` gate columns, their `strip` up columns, and so on.  bias: float32 [2*inter] in the
-    rows' own column order, added before the activation."""
+    "gelu_tanh"; or "clamped_swish": with g = min(gate, limit) and u = clamp(up, -limit, limit),
+    out = g sigmoid(alpha g) (u + 1).  strip = 0: the gate columns come first, then the up
+    columns; strip > 0: `strip` gate columns, their `strip` up columns, and so on.  bias:
+    float32 [2*inter] in the rows' own column order, added before the activation."""
     lib = library("rowwise")
     if activation not in GATE_ACTIVATIONS:
         raise KernelError(f"swiglu: unknown gate activation '{activation}'; "
@@ -322,8 +350,43 @@ def swiglu(gate_up: torch.Tensor, out: torch.Tensor, strip: int = 0,
     status = lib.ei_swiglu(_gpu(gate_up, "gate_up"), _code(gate_up, "gate_up"), nsplit, stride,
                            _gpu(out, "out"), _code(out, "out"), n, inter, int(strip),
                            GATE_ACTIVATIONS[activation],
-                           None if bias is None else _gpu(bias, "bias", torch.float32), _stream())
+                           None if bias is None else _gpu(bias, "bias", torch.float32),
+                           float(limit), float(alpha), _stream())
     _check(lib, status, "swiglu")
+
+
+def norm_rows(x: torch.Tensor, weight: torch.Tensor, eps: float) -> None:
+    """x [rows, H] float32 <- x / sqrt(mean(x^2) + eps) * weight, in place."""
+    lib = library("rowwise")
+    rows, hidden = x.shape
+    if weight.numel() != hidden:
+        raise KernelError("norm_rows: the weight must be as wide as a row")
+    status = lib.ei_norm_rows(_gpu(x, "x", torch.float32), _gpu(weight, "weight", torch.float32),
+                              float(eps), rows, hidden, _stream())
+    _check(lib, status, "norm_rows")
+
+
+def gate_rows(gate: torch.Tensor, first_column: int, out: torch.Tensor) -> None:
+    """out [n, w] *= sigmoid(gate[:, first_column : first_column + w]) for gate [n, g] in out's
+    type or float32, or float32 slices [s, n, g] (summed first)."""
+    lib = library("rowwise")
+    n, width = out.shape
+    stride = gate.shape[-1]
+    nsplit, split_stride = _splits(gate, n, stride, "gate")
+    if not 0 <= first_column <= stride - width:
+        raise KernelError("gate_rows: the gate's columns lie outside its rows")
+    status = lib.ei_gate_rows(_gpu(gate, "gate"), _code(gate, "gate"), nsplit, split_stride,
+                              stride, int(first_column), _gpu(out, "out"), _code(out, "out"), n,
+                              width, _stream())
+    _check(lib, status, "gate_rows")
+
+
+def scale_cap(x: torch.Tensor, scale: float, cap: Optional[float]) -> None:
+    """x (float32) <- cap tanh(scale x / cap), or scale x without a cap, in place."""
+    lib = library("rowwise")
+    status = lib.ei_scale_cap(_gpu(x, "x", torch.float32), float(scale), float(cap or 0.0),
+                              x.numel(), _stream())
+    _check(lib, status, "scale_cap")
 
 
 def sum_slices(slices: torch.Tensor, out: torch.Tensor) -> None:
@@ -839,6 +902,62 @@ def projection_norm_store(qkv, q_norm_w, k_norm_w, eps, row_pos, row_seq, page_t
     _check(lib, status, "projection_norm_store")
 
 
+def head_store(proj, q_norm_w, k_norm_w, eps, frequencies, row_pos, row_seq, page_table, q_out,
+               k_pages, v_pages, n_heads, n_kv_heads, head_dim, value_dim, write_cache=True,
+               v_first=None, v_mode=0, v_lambda=None) -> None:
+    """Rows that begin with [q | k | v] (and may go on with other columns), as [n, g] or float32
+    slices [s, n, g]: per-head RMS norm of queries and keys (weights [head_dim], or None), the
+    rotation of every head's first R elements in pairs (i, i + R/2) by float(position) *
+    frequencies[i] (float32 [R/2], or None for no rotation), queries to `q_out`, keys
+    [*, kv heads, 64, head_dim] and values [*, kv heads, 64, value_dim] to their pages.
+    v_mode 1: the values are also written to `v_first` (float32 [n, kv heads * value_dim]);
+    v_mode 2: what is stored is (1 - lambda) v + lambda v_first, `v_lambda` one float32 on the
+    device."""
+    lib = library("rope_store")
+    n = q_out.shape[0]
+    stride = proj.shape[-1]
+    nsplit, split_stride = _splits(proj, n, stride, "proj")
+    if stride < n_heads * head_dim + n_kv_heads * (head_dim + value_dim):
+        raise KernelError("head_store: the rows are narrower than the projections")
+    if tuple(q_out.shape) != (n, n_heads * head_dim):
+        raise KernelError("head_store: q_out has the wrong shape")
+    if row_pos.numel() < n or row_seq.numel() < n:
+        raise KernelError("head_store: row metadata shorter than the rows")
+    for weight in (q_norm_w, k_norm_w):
+        if weight is not None and weight.numel() != head_dim:
+            raise KernelError("head_store: a norm weight must be as wide as a head")
+    rot_dim = 0
+    if frequencies is not None:
+        rot_dim = 2 * frequencies.numel()
+        if frequencies.dim() != 1 or not 2 <= rot_dim <= head_dim:
+            raise KernelError("head_store: the frequencies must be [R/2] with R at most head_dim")
+    if write_cache:
+        if tuple(k_pages.shape[1:]) != (n_kv_heads, PAGE_TOKENS, head_dim) or \
+                tuple(v_pages.shape) != (k_pages.shape[0], n_kv_heads, PAGE_TOKENS, value_dim):
+            raise KernelError("head_store: pages have the wrong shape")
+        if k_pages.dtype != q_out.dtype or v_pages.dtype != q_out.dtype:
+            raise KernelError("head_store: cache and q_out dtypes differ")
+    if v_mode not in (0, 1, 2):
+        raise KernelError("head_store: v_mode must be 0, 1 or 2")
+    if v_mode and (v_first is None or tuple(v_first.shape) != (n, n_kv_heads * value_dim)):
+        raise KernelError("head_store: v_first must be float32 [rows, kv heads * value_dim]")
+    if v_mode == 2 and (v_lambda is None or v_lambda.numel() != 1):
+        raise KernelError("head_store: mixing values needs its one weight")
+    status = lib.ei_head_store(
+        _gpu(proj, "proj"), _code(proj, "proj"), nsplit, split_stride, stride,
+        None if q_norm_w is None else _gpu(q_norm_w, "q_norm", torch.float32),
+        None if k_norm_w is None else _gpu(k_norm_w, "k_norm", torch.float32), float(eps),
+        None if frequencies is None else _gpu(frequencies, "frequencies", torch.float32), rot_dim,
+        _gpu(row_pos, "row_pos", torch.int32), _gpu(row_seq, "row_seq", torch.int32),
+        _gpu(page_table, "page_table", torch.int32), page_table.shape[-1], _gpu(q_out, "q_out"),
+        _gpu(k_pages, "k_pages") if write_cache else None,
+        _gpu(v_pages, "v_pages") if write_cache else None, _code(q_out, "q_out"),
+        None if not v_mode else _gpu(v_first, "v_first", torch.float32), int(v_mode),
+        None if v_mode != 2 else _gpu(v_lambda, "v_lambda", torch.float32), n, n_heads,
+        n_kv_heads, head_dim, value_dim, int(write_cache), _stream())
+    _check(lib, status, "head_store")
+
+
 MFMA_HEAD_DIMS = (64, 128)
 
 
@@ -1154,6 +1273,158 @@ def delta_out(o_raw, proj, norm_w, eps, shape: DeltaShape, row_seq, out) -> None
     _check(lib, status, "delta_out")
 
 
+# ---------------------------------------------------------------------------
+class SsmShape:
+    """Sizes of a state-space mixer: heads of `head_dim` columns each, `groups` pairs of B and C
+    vectors of `state` elements, `taps` of the convolution.  A projection row is
+    [z: inner | x: inner | B: groups * state | C: groups * state | dt: heads]."""
+
+    def __init__(self, heads, groups, head_dim, state, taps):
+        self.heads, self.groups, self.head_dim = int(heads), int(groups), int(head_dim)
+        self.state, self.taps = int(state), int(taps)
+        self.inner = self.heads * self.head_dim
+        self.channels = self.inner + 2 * self.groups * self.state      # what is convolved
+        self.proj_width = self.inner + self.channels + self.heads
+        # S of every head [head][column][row], then the convolution's last taps - 1 inputs
+        self.state_floats = self.inner * self.state + (self.taps - 1) * self.channels
+
+    @property
+    def sizes(self):
+        return (self.heads, self.groups, self.head_dim, self.state, self.taps)
+
+
+def _ssm_proj(proj, rows, shape):
+    if proj.shape[-1] != shape.proj_width:
+        raise KernelError(f"ssm: the projection must be {shape.proj_width} wide")
+    return _splits(proj, rows, shape.proj_width, "proj")
+
+
+def _ssm_state(state, shape):
+    if state.dim() != 2 or state.shape[1] != shape.state_floats:
+        raise KernelError(f"ssm: the state table must be [rows, {shape.state_floats}]")
+    return _gpu(state, "state", torch.float32)
+
+
+def ssm_conv(proj, conv_w, conv_b, state, shape: SsmShape, row_pos, row_seq, seq_in, seq_out,
+             seq_start, seq_count, seq_row0, conv) -> None:
+    """conv [n, channels] float32 = silu(causal convolution of the x, B and C columns of `proj`
+    + bias), earlier inputs taken from the step's rows or the sequence's tail in row
+    `seq_in[s]` of `state`; the new tails are written to row `seq_out[s]`."""
+    lib = library("ssm")
+    n = conv.shape[0]
+    nsplit, stride = _ssm_proj(proj, n, shape)
+    n_seqs = seq_in.numel()
+    if tuple(conv.shape) != (n, shape.channels) or tuple(conv_w.shape) != (shape.channels, shape.taps):
+        raise KernelError("ssm_conv: conv or its filters have the wrong shape")
+    if conv_b is not None and conv_b.numel() != shape.channels:
+        raise KernelError("ssm_conv: the bias must have one value a channel")
+    if row_pos.numel() < n or row_seq.numel() < n or min(
+            seq_out.numel(), seq_start.numel(), seq_count.numel(), seq_row0.numel()) < n_seqs:
+        raise KernelError("ssm_conv: metadata shorter than the step")
+    status = lib.ei_ssm_conv(
+        _gpu(proj, "proj"), _code(proj, "proj"), nsplit, stride, shape.proj_width,
+        _gpu(conv_w, "conv_w", torch.float32),
+        None if conv_b is None else _gpu(conv_b, "conv_b", torch.float32),
+        _ssm_state(state, shape), state.shape[1], _gpu(row_pos, "row_pos", torch.int32),
+        _gpu(row_seq, "row_seq", torch.int32), _gpu(seq_in, "seq_in", torch.int32),
+        _gpu(seq_out, "seq_out", torch.int32), _gpu(seq_start, "seq_start", torch.int32),
+        _gpu(seq_count, "seq_count", torch.int32), _gpu(seq_row0, "seq_row0", torch.int32),
+        _gpu(conv, "conv", torch.float32), n, n_seqs, *shape.sizes, _stream())
+    _check(lib, status, "ssm_conv")
+
+
+def ssm_scan(conv, proj, a_log, dt_bias, d_skip, state, shape: SsmShape, seq_in, seq_out,
+             seq_count, seq_row0, y_raw) -> None:
+    """The recurrence over every sequence's rows: S <- exp(-exp(a_log) dt) S + dt B x^T from row
+    `seq_in[s]` of `state`, y = S^T C + d_skip x to `y_raw` [n, inner] float32, the last S to row
+    `seq_out[s]`; dt = softplus(proj's dt column + dt_bias)."""
+    lib = library("ssm")
+    n = y_raw.shape[0]
+    nsplit, stride = _ssm_proj(proj, n, shape)
+    n_seqs = seq_in.numel()
+    if tuple(conv.shape) != (n, shape.channels) or tuple(y_raw.shape) != (n, shape.inner):
+        raise KernelError("ssm_scan: conv or y_raw has the wrong shape")
+    for name, per_head in (("a_log", a_log), ("dt_bias", dt_bias), ("d_skip", d_skip)):
+        if per_head.numel() != shape.heads:
+            raise KernelError(f"ssm_scan: {name} must have one value a head")
+    if min(seq_out.numel(), seq_count.numel(), seq_row0.numel()) < n_seqs:
+        raise KernelError("ssm_scan: metadata shorter than the step")
+    status = lib.ei_ssm_scan(
+        _gpu(conv, "conv", torch.float32), _gpu(proj, "proj"), _code(proj, "proj"), nsplit, stride,
+        shape.proj_width, _gpu(a_log, "a_log", torch.float32),
+        _gpu(dt_bias, "dt_bias", torch.float32), _gpu(d_skip, "d_skip", torch.float32),
+        _ssm_state(state, shape), state.shape[1], _gpu(seq_in, "seq_in", torch.int32),
+        _gpu(seq_out, "seq_out", torch.int32), _gpu(seq_count, "seq_count", torch.int32),
+        _gpu(seq_row0, "seq_row0", torch.int32), _gpu(y_raw, "y_raw", torch.float32), n_seqs,
+        *shape.sizes, _stream())
+    _check(lib, status, "ssm_scan")
+
+
+def ssm_out(y_raw, proj, norm_w, eps, shape: SsmShape, parts, row_seq, out) -> None:
+    """out [n, inner] = rmsnorm over each of `parts` equal parts of (y_raw * silu(z)) * norm_w,
+    z the first `inner` columns of `proj`."""
+    lib = library("ssm")
+    n = out.shape[0]
+    nsplit, stride = _ssm_proj(proj, n, shape)
+    if tuple(y_raw.shape) != (n, shape.inner) or tuple(out.shape) != (n, shape.inner):
+        raise KernelError("ssm_out: y_raw and out must be [rows, inner]")
+    if norm_w.numel() != shape.inner or parts < 1 or shape.inner % parts:
+        raise KernelError("ssm_out: the weight must be [inner] and the parts divide it")
+    status = lib.ei_ssm_out(_gpu(y_raw, "y_raw", torch.float32), _gpu(proj, "proj"),
+                            _code(proj, "proj"), nsplit, stride, shape.proj_width,
+                            _gpu(norm_w, "norm_w", torch.float32), float(eps),
+                            _gpu(row_seq, "row_seq", torch.int32), _gpu(out, "out"),
+                            _code(out, "out"), n, shape.inner, int(parts), _stream())
+    _check(lib, status, "ssm_out")
+
+
+# ---------------------------------------------------------------------------
+def moe_route(x, router_w, row_seq, expert, weight) -> None:
+    """For every row of x [n, w]: the `top` experts of largest float32 logit router_w [E, w] . x
+    into `expert` (int32 [n, top], largest first), the softmax over their logits into `weight`
+    (float32 [n, top]).  Rows with row_seq < 0 get weights of 0."""
+    lib = library("moe")
+    n, width = x.shape
+    n_experts = router_w.shape[0]
+    top = expert.shape[1]
+    if tuple(router_w.shape) != (n_experts, width) or tuple(expert.shape) != (n, top) \
+            or tuple(weight.shape) != (n, top):
+        raise KernelError("moe_route: shapes do not fit")
+    if row_seq is not None and row_seq.numel() < n:
+        raise KernelError("moe_route: row metadata shorter than the rows")
+    status = lib.ei_moe_route(_gpu(x, "x"), _code(x, "x"), _gpu(router_w, "router_w", torch.float32),
+                              None if row_seq is None else _gpu(row_seq, "row_seq", torch.int32),
+                              _gpu(expert, "expert", torch.int32),
+                              _gpu(weight, "weight", torch.float32), n, width, n_experts, top,
+                              _stream())
+    _check(lib, status, "moe_route")
+
+
+def moe_experts(x, w_gate, w_up, w_down, expert, weight, act, out) -> None:
+    """out [n, w] float32 = sum over a row's choices k of weight[r, k] *
+    w_down[e] (silu(w_gate[e] x_r) * (w_up[e] x_r)), e = expert[r, k]; w_gate and w_up
+    [E, f, w], w_down [E, w, f], all of x's type; `act` [n * top, f] of that type is scratch."""
+    lib = library("moe")
+    n, width = x.shape
+    n_experts, inter = w_gate.shape[0], w_gate.shape[1]
+    top = expert.shape[1]
+    if tuple(w_gate.shape) != (n_experts, inter, width) or tuple(w_up.shape) != tuple(w_gate.shape) \
+            or tuple(w_down.shape) != (n_experts, width, inter):
+        raise KernelError("moe_experts: the stacked matrices have the wrong shapes")
+    if tuple(expert.shape) != (n, top) or tuple(weight.shape) != (n, top) \
+            or tuple(act.shape) != (n * top, inter) or tuple(out.shape) != (n, width):
+        raise KernelError("moe_experts: shapes do not fit")
+    if not (x.dtype == w_gate.dtype == w_up.dtype == w_down.dtype == act.dtype):
+        raise KernelError("moe_experts: x, the matrices and act must have one type")
+    status = lib.ei_moe_experts(_gpu(x, "x"), _gpu(w_gate, "w_gate"), _gpu(w_up, "w_up"),
+                                _gpu(w_down, "w_down"), _code(x, "x"),
+                                _gpu(expert, "expert", torch.int32),
+                                _gpu(weight, "weight", torch.float32), _gpu(act, "act"),
+                                _gpu(out, "out", torch.float32), n, width, inter, top, _stream())
+    _check(lib, status, "moe_experts")
+
+
+# ---------------------------------------------------------------------------
 def gemm_f32(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
     """out[M, N] = a[M, K] . w[N, K]^T in float32."""
     lib = library("gemm_f32")

@@ -613,3 +613,142 @@ extern "C" int ei_projection_norm_store(
 #undef EI_PNS_V
   EI_LAUNCH_CHECK();
 }
+
+// ---------------------------------------------------------------------------------------
+// The store for heads whose values have a width of their own, whose rotation works out its
+// angles from frequencies (angle = float(position) * f_i in float32, cosine and sine taken
+// here: no table, no longest position), and whose values may be mixed with the values that
+// an earlier layer of the same step computed for the same token.
+//
+// proj: rows `row_stride` wide that begin with [q: nq * D | k: nkv * D | v: nkv * DV]
+// (whatever follows is another kernel's).  One wave a (row, head).  Query and key heads:
+// optional RMS norm over the head with a weight [D], then the rotation of the first R
+// elements in pairs (i, i + R/2), then queries to q_out and keys to their page.  Value heads:
+// v_mode 0: stored as they are; 1: also written, in float32, to v_first [N, nkv * DV];
+// 2: v <- (1 - lambda) v + lambda v_first before the store (lambda one float on the device).
+namespace {
+
+constexpr int kHeadStoreMax = 8;  // elements a lane: head sizes up to 512
+
+template <typename TI>
+__device__ __forceinline__ float sliced(const TI* p, int nsplit, size_t split_stride) {
+  float v = 0.f;
+  for (int s = 0; s < nsplit; ++s) v += ei::to_f32<TI>(p[s * split_stride]);
+  return v;
+}
+
+template <typename TI, typename TO>
+__global__ void head_store_kernel(
+    const TI* __restrict__ proj, int nsplit, size_t split_stride, size_t row_stride,
+    const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w, float eps,
+    const float* __restrict__ freqs, int R, const int32_t* __restrict__ row_pos,
+    const int32_t* __restrict__ row_seq, const int32_t* __restrict__ page_table, int table_width,
+    TO* __restrict__ q_out, TO* __restrict__ k_pages, TO* __restrict__ v_pages,
+    float* __restrict__ v_first, int v_mode, const float* __restrict__ v_lambda,
+    int N, int nq, int nkv, int D, int DV, int write_cache) {
+  const int heads = nq + 2 * nkv;
+  const int wave = (blockIdx.x * blockDim.x + threadIdx.x) / EI_WAVE;
+  const int lane = threadIdx.x % EI_WAVE;
+  if (wave >= N * heads) return;
+  const int row = wave / heads, head = wave % heads;
+  const int seq = row_seq[row];
+  if (seq < 0) return;  // padding row
+  const int pos = row_pos[row];
+  const TI* src_row = proj + static_cast<size_t>(row) * row_stride;
+  size_t page_slot = 0;   // (page, position in the page) of this row, if the cache is written
+  if (write_cache)
+    page_slot = static_cast<size_t>(page_table[static_cast<size_t>(seq) * table_width + pos / EI_PAGE]);
+
+  if (head >= nq + nkv) {   // a value head
+    const int h = head - nq - nkv;
+    const TI* src = src_row + static_cast<size_t>(nq + nkv) * D + static_cast<size_t>(h) * DV;
+    float* first = v_first ? v_first + static_cast<size_t>(row) * nkv * DV + static_cast<size_t>(h) * DV
+                           : nullptr;
+    const float lambda = v_mode == 2 ? *v_lambda : 0.f;
+    TO* dst = write_cache
+                  ? v_pages + ((page_slot * nkv + h) * EI_PAGE + pos % EI_PAGE) * static_cast<size_t>(DV)
+                  : nullptr;
+    for (int e = lane; e < DV; e += EI_WAVE) {
+      float v = sliced(src + e, nsplit, split_stride);
+      if (v_mode == 1) first[e] = v;
+      else if (v_mode == 2) v = (1.0f - lambda) * v + lambda * first[e];
+      if (dst) dst[e] = ei::from_f32<TO>(v);
+    }
+    return;
+  }
+  const bool is_q = head < nq;
+  if (!is_q && !write_cache) return;
+  const TI* src = src_row + static_cast<size_t>(head) * D;
+  const float* w = is_q ? q_norm_w : k_norm_w;
+  const int rhalf = R / 2;
+  float x[kHeadStoreMax], y[kHeadStoreMax];   // a lane's elements and their partners in the rotation
+  float sum = 0.f;
+#pragma unroll
+  for (int j = 0; j < kHeadStoreMax; ++j) {
+    const int e = lane + j * EI_WAVE;
+    x[j] = y[j] = 0.f;
+    if (e < D) {
+      x[j] = sliced(src + e, nsplit, split_stride);
+      sum += x[j] * x[j];
+      if (e < R) y[j] = sliced(src + (e < rhalf ? e + rhalf : e - rhalf), nsplit, split_stride);
+    }
+  }
+  float inv = 1.0f;
+  if (w) inv = 1.0f / sqrtf(ei::wave_sum(sum) / static_cast<float>(D) + eps);
+  TO* dst = is_q ? q_out + (static_cast<size_t>(row) * nq + head) * D
+                 : k_pages + ((page_slot * nkv + (head - nq)) * EI_PAGE + pos % EI_PAGE) * static_cast<size_t>(D);
+#pragma unroll
+  for (int j = 0; j < kHeadStoreMax; ++j) {
+    const int e = lane + j * EI_WAVE;
+    if (e >= D) continue;
+    float v = w ? (x[j] * inv) * w[e] : x[j];
+    if (e < R) {
+      const int partner = e < rhalf ? e + rhalf : e - rhalf;
+      const float p = w ? (y[j] * inv) * w[partner] : y[j];
+      const float angle = static_cast<float>(pos) * freqs[e < rhalf ? e : e - rhalf];
+      float sn, cs;
+      sincosf(angle, &sn, &cs);
+      v = e < rhalf ? v * cs - p * sn : v * cs + p * sn;
+    }
+    dst[e] = ei::from_f32<TO>(v);
+  }
+}
+
+}  // namespace
+
+extern "C" int ei_head_store(
+    const void* proj, int in_dtype, int nsplit, long long split_stride, long long row_stride,
+    const float* q_norm_w, const float* k_norm_w, float eps, const float* freqs, int rot_dim,
+    const int32_t* row_pos, const int32_t* row_seq, const int32_t* page_table, int table_width,
+    void* q_out, void* k_pages, void* v_pages, int out_dtype, float* v_first, int v_mode,
+    const float* v_lambda, int N, int nq, int nkv, int D, int DV, int write_cache,
+    hipStream_t stream) {
+  EI_REQUIRE(N > 0 && nq > 0 && nkv > 0 && D > 0 && DV > 0, "head_store: sizes must be positive");
+  EI_REQUIRE(D <= kHeadStoreMax * EI_WAVE, "head_store: head_dim above 512");
+  EI_REQUIRE(proj && row_pos && row_seq && q_out && nsplit >= 1, "head_store: bad arguments");
+  EI_REQUIRE(row_stride >= static_cast<long long>(nq + nkv) * D + static_cast<long long>(nkv) * DV,
+             "head_store: rows narrower than the projections");
+  EI_REQUIRE(!write_cache || (k_pages && v_pages && page_table && table_width > 0),
+             "head_store: cache pointers missing");
+  EI_REQUIRE((q_norm_w == nullptr) == (k_norm_w == nullptr), "head_store: both norm weights or neither");
+  const int R = freqs ? rot_dim : 0;
+  EI_REQUIRE(R % 2 == 0 && R >= 0 && R <= D, "head_store: the rotated width must be even and at most head_dim");
+  EI_REQUIRE(v_mode >= 0 && v_mode <= 2 && (v_mode == 0 || v_first) && (v_mode != 2 || v_lambda),
+             "head_store: value mixing needs its buffer and its weight");
+  const int heads = nq + 2 * nkv;
+  const int threads = 256;
+  const size_t waves = static_cast<size_t>(N) * heads;
+  const unsigned blocks = static_cast<unsigned>((waves * EI_WAVE + threads - 1) / threads);
+  const size_t ss = static_cast<size_t>(split_stride), rs = static_cast<size_t>(row_stride);
+#define EI_HS(TI, TO)                                                                          \
+  head_store_kernel<TI, TO><<<blocks, threads, 0, stream>>>(                                   \
+      static_cast<const TI*>(proj), nsplit, ss, rs, q_norm_w, k_norm_w, eps, freqs, R, row_pos, \
+      row_seq, page_table, table_width, static_cast<TO*>(q_out), static_cast<TO*>(k_pages),    \
+      static_cast<TO*>(v_pages), v_first, v_mode, v_lambda, N, nq, nkv, D, DV, write_cache)
+  if (in_dtype == EI_F32 && out_dtype == EI_F32) EI_HS(float, float);
+  else if (in_dtype == EI_F32 && out_dtype == EI_BF16) EI_HS(float, bf16_t);
+  else if (in_dtype == EI_BF16 && out_dtype == EI_BF16) EI_HS(bf16_t, bf16_t);
+  else EI_REQUIRE(false, "head_store: unsupported dtype combination");
+#undef EI_HS
+  EI_LAUNCH_CHECK();
+}

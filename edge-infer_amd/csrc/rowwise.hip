@@ -137,10 +137,20 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ residual, const TD* _
 
 // Where gate and up of output column `col` lie in a row of 2I: the halves [gate | up]
 // (strip = 0), or strips of `strip` gate columns followed by their `strip` up columns.
-// gate activations of the C interface: 0 silu, 1 the tanh form of gelu
+// gate activations of the C interface: 0 silu, 1 the tanh form of gelu, 2 the clamped swish:
+// with g = min(gate, limit) and u = clamp(up, -limit, limit) the product is
+// g sigmoid(alpha g) (u + 1)
 template <typename TO> __device__ __forceinline__ float gate_act(float x, int act) {
   if (act == 0) return ei::silu<TO>(x);
   return 0.5f * x * (1.0f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x)));
+}
+
+template <typename TO>
+__device__ __forceinline__ float gated_product(float gate, float up, int act, float limit, float alpha) {
+  if (act != 2) return gate_act<TO>(gate, act) * up;
+  const float g = fminf(gate, limit);
+  const float u = fminf(fmaxf(up, -limit), limit);
+  return g / (1.0f + expf(-alpha * g)) * (u + 1.0f);
 }
 
 __device__ __forceinline__ size_t gate_column(size_t col, int strip) {
@@ -150,7 +160,7 @@ __device__ __forceinline__ size_t gate_column(size_t col, int strip) {
 template <typename TI, typename TO>
 __global__ void swiglu_kernel(const TI* __restrict__ gate_up, int nsplit, size_t split_stride,
                               TO* __restrict__ out, int I, size_t total, int strip, int act,
-                              const float* __restrict__ bias) {
+                              const float* __restrict__ bias, float limit, float alpha) {
   const size_t start = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   const size_t step = static_cast<size_t>(gridDim.x) * blockDim.x;
   const size_t up_offset = strip ? strip : I;
@@ -166,7 +176,7 @@ __global__ void swiglu_kernel(const TI* __restrict__ gate_up, int nsplit, size_t
       gate += bias[gate_column(col, strip)];
       up += bias[gate_column(col, strip) + up_offset];
     }
-    out[idx] = ei::from_f32<TO>(gate_act<TO>(gate, act) * up);
+    out[idx] = ei::from_f32<TO>(gated_product<TO>(gate, up, act, limit, alpha));
   }
 }
 
@@ -175,7 +185,7 @@ __global__ void swiglu_kernel(const TI* __restrict__ gate_up, int nsplit, size_t
 template <typename TI, typename TO>
 __global__ void swiglu_vec_kernel(const TI* __restrict__ gate_up, int nsplit, size_t split_stride,
                                   TO* __restrict__ out, int I, size_t total_octets, int strip, int act,
-                                  const float* __restrict__ bias) {
+                                  const float* __restrict__ bias, float limit, float alpha) {
   const size_t start = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   const size_t step = static_cast<size_t>(gridDim.x) * blockDim.x;
   const int octets_per_row = I / 8;
@@ -221,8 +231,8 @@ __global__ void swiglu_vec_kernel(const TI* __restrict__ gate_up, int nsplit, si
     float y0[4], y1[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      y0[i] = gate_act<TO>(gate[i], act) * up[i];
-      y1[i] = gate_act<TO>(gate[i + 4], act) * up[i + 4];
+      y0[i] = gated_product<TO>(gate[i], up[i], act, limit, alpha);
+      y1[i] = gated_product<TO>(gate[i + 4], up[i + 4], act, limit, alpha);
     }
     TO* dst = out + row * I + col;
     Vec4<TO>::store(dst, y0);
@@ -369,9 +379,9 @@ extern "C" int ei_add_rmsnorm(float* residual, const void* delta, int delta_dtyp
 // strip > 0 (a divisor of I): `strip` gate columns, their `strip` up columns, and so on.
 extern "C" int ei_swiglu(const void* gate_up, int in_dtype, int nsplit, long long split_stride,
                          void* out, int out_dtype, int N, int I, int strip, int act,
-                         const float* bias, hipStream_t stream) {
+                         const float* bias, float limit, float alpha, hipStream_t stream) {
   EI_REQUIRE(N > 0 && I > 0 && nsplit >= 1, "swiglu: sizes must be positive");
-  EI_REQUIRE(act == 0 || act == 1, "swiglu: unknown gate activation");
+  EI_REQUIRE(act >= 0 && act <= 2, "swiglu: unknown gate activation");
   EI_REQUIRE(gate_up && out, "swiglu: null pointer");
   EI_REQUIRE(strip >= 0 && (strip == 0 || I % strip == 0), "swiglu: the strip must divide the width");
   const size_t total = static_cast<size_t>(N) * I;
@@ -383,13 +393,13 @@ extern "C" int ei_swiglu(const void* gate_up, int in_dtype, int nsplit, long lon
     if (vblocks > ei_compute_units() * 32) vblocks = ei_compute_units() * 32;
     if (in_dtype == EI_F32 && out_dtype == EI_F32)
       swiglu_vec_kernel<float, float><<<vblocks, threads, 0, stream>>>(
-          static_cast<const float*>(gate_up), nsplit, ss, static_cast<float*>(out), I, octets, strip, act, bias);
+          static_cast<const float*>(gate_up), nsplit, ss, static_cast<float*>(out), I, octets, strip, act, bias, limit, alpha);
     else if (in_dtype == EI_F32 && out_dtype == EI_BF16)
       swiglu_vec_kernel<float, bf16_t><<<vblocks, threads, 0, stream>>>(
-          static_cast<const float*>(gate_up), nsplit, ss, static_cast<bf16_t*>(out), I, octets, strip, act, bias);
+          static_cast<const float*>(gate_up), nsplit, ss, static_cast<bf16_t*>(out), I, octets, strip, act, bias, limit, alpha);
     else if (in_dtype == EI_BF16 && out_dtype == EI_BF16)
       swiglu_vec_kernel<bf16_t, bf16_t><<<vblocks, threads, 0, stream>>>(
-          static_cast<const bf16_t*>(gate_up), nsplit, ss, static_cast<bf16_t*>(out), I, octets, strip, act, bias);
+          static_cast<const bf16_t*>(gate_up), nsplit, ss, static_cast<bf16_t*>(out), I, octets, strip, act, bias, limit, alpha);
     else
       EI_REQUIRE(false, "swiglu: unsupported dtype combination");
     EI_LAUNCH_CHECK();
@@ -398,13 +408,13 @@ extern "C" int ei_swiglu(const void* gate_up, int in_dtype, int nsplit, long lon
   if (blocks > ei_compute_units() * 32) blocks = ei_compute_units() * 32;
   if (in_dtype == EI_F32 && out_dtype == EI_F32)
     swiglu_kernel<float, float><<<blocks, threads, 0, stream>>>(
-        static_cast<const float*>(gate_up), nsplit, ss, static_cast<float*>(out), I, total, strip, act, bias);
+        static_cast<const float*>(gate_up), nsplit, ss, static_cast<float*>(out), I, total, strip, act, bias, limit, alpha);
   else if (in_dtype == EI_F32 && out_dtype == EI_BF16)
     swiglu_kernel<float, bf16_t><<<blocks, threads, 0, stream>>>(
-        static_cast<const float*>(gate_up), nsplit, ss, static_cast<bf16_t*>(out), I, total, strip, act, bias);
+        static_cast<const float*>(gate_up), nsplit, ss, static_cast<bf16_t*>(out), I, total, strip, act, bias, limit, alpha);
   else if (in_dtype == EI_BF16 && out_dtype == EI_BF16)
     swiglu_kernel<bf16_t, bf16_t><<<blocks, threads, 0, stream>>>(
-        static_cast<const bf16_t*>(gate_up), nsplit, ss, static_cast<bf16_t*>(out), I, total, strip, act, bias);
+        static_cast<const bf16_t*>(gate_up), nsplit, ss, static_cast<bf16_t*>(out), I, total, strip, act, bias, limit, alpha);
   else
     EI_REQUIRE(false, "swiglu: unsupported dtype combination");
   EI_LAUNCH_CHECK();
@@ -901,5 +911,88 @@ extern "C" int ei_set_rows(const void* x, int x_dtype, int nsplit, long long spl
         static_cast<const bf16_t*>(x), nsplit, ss, vec, out, H, n);
   else
     EI_REQUIRE(false, "set_rows: unknown dtype");
+  EI_LAUNCH_CHECK();
+}
+
+// ---------------------------------------------------------------------------------------
+// x [rows, H] float32 <- x / sqrt(mean(x^2) + eps) * w, in place: a norm that sits on the
+// stream itself (the one behind an embedding).  A block a row.
+namespace {
+__global__ void norm_rows_kernel(float* __restrict__ x, const float* __restrict__ w, float eps, int H) {
+  __shared__ float scratch[16];
+  float* row = x + static_cast<size_t>(blockIdx.x) * H;
+  float sum = 0.f;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) sum += row[i] * row[i];
+  const float inv = 1.0f / sqrtf(ei::block_sum(sum, scratch) / static_cast<float>(H) + eps);
+  for (int i = threadIdx.x; i < H; i += blockDim.x) row[i] = (row[i] * inv) * w[i];
+}
+
+// out [rows, W] *= sigmoid(gate), gate the columns col0 .. col0 + W - 1 of rows `stride` wide
+// (or the sum of `nsplit` float32 slices of them).
+template <typename TG, typename TO>
+__global__ void gate_rows_kernel(const TG* __restrict__ gate, int nsplit, size_t split_stride,
+                                 size_t stride, int col0, TO* __restrict__ out, int W, size_t total) {
+  const size_t start = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const size_t step = static_cast<size_t>(gridDim.x) * blockDim.x;
+  for (size_t idx = start; idx < total; idx += step) {
+    const size_t row = idx / W, col = idx % W;
+    const TG* g = gate + row * stride + col0 + col;
+    float z = 0.f;
+    for (int s = 0; s < nsplit; ++s) z += ei::to_f32<TG>(g[s * split_stride]);
+    out[idx] = ei::from_f32<TO>(ei::to_f32<TO>(out[idx]) / (1.0f + expf(-z)));
+  }
+}
+
+// x <- cap tanh(scale x / cap) (cap > 0), or scale x.
+__global__ void scale_cap_kernel(float* __restrict__ x, float scale, float cap, size_t total) {
+  const size_t start = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const size_t step = static_cast<size_t>(gridDim.x) * blockDim.x;
+  for (size_t i = start; i < total; i += step) {
+    const float v = x[i] * scale;
+    x[i] = cap > 0.f ? cap * tanhf(v / cap) : v;
+  }
+}
+}  // namespace
+
+extern "C" int ei_norm_rows(float* x, const float* w, float eps, long long rows, int H,
+                            hipStream_t stream) {
+  EI_REQUIRE(x && w && rows > 0 && H > 0, "norm_rows: bad arguments");
+  const int threads = H >= 1024 ? 256 : (H >= 256 ? 128 : 64);
+  norm_rows_kernel<<<static_cast<unsigned>(rows), threads, 0, stream>>>(x, w, eps, H);
+  EI_LAUNCH_CHECK();
+}
+
+extern "C" int ei_gate_rows(const void* gate, int gate_dtype, int nsplit, long long split_stride,
+                            long long stride, int col0, void* out, int out_dtype, long long rows,
+                            int W, hipStream_t stream) {
+  EI_REQUIRE(gate && out && rows > 0 && W > 0 && nsplit >= 1 && col0 >= 0 && col0 + W <= stride,
+             "gate_rows: bad arguments");
+  const size_t total = static_cast<size_t>(rows) * W;
+  const int threads = 256;
+  size_t blocks = (total + threads - 1) / threads;
+  if (blocks > ei_compute_units() * 16) blocks = ei_compute_units() * 16;
+  const size_t ss = static_cast<size_t>(split_stride), st = static_cast<size_t>(stride);
+  const unsigned b = static_cast<unsigned>(blocks);
+  if (gate_dtype == EI_F32 && out_dtype == EI_F32)
+    gate_rows_kernel<float, float><<<b, threads, 0, stream>>>(
+        static_cast<const float*>(gate), nsplit, ss, st, col0, static_cast<float*>(out), W, total);
+  else if (gate_dtype == EI_F32 && out_dtype == EI_BF16)
+    gate_rows_kernel<float, bf16_t><<<b, threads, 0, stream>>>(
+        static_cast<const float*>(gate), nsplit, ss, st, col0, static_cast<bf16_t*>(out), W, total);
+  else if (gate_dtype == EI_BF16 && out_dtype == EI_BF16)
+    gate_rows_kernel<bf16_t, bf16_t><<<b, threads, 0, stream>>>(
+        static_cast<const bf16_t*>(gate), nsplit, ss, st, col0, static_cast<bf16_t*>(out), W, total);
+  else
+    EI_REQUIRE(false, "gate_rows: unsupported dtype combination");
+  EI_LAUNCH_CHECK();
+}
+
+extern "C" int ei_scale_cap(float* x, float scale, float cap, long long total, hipStream_t stream) {
+  EI_REQUIRE(x && total > 0, "scale_cap: bad arguments");
+  const int threads = 256;
+  size_t blocks = (static_cast<size_t>(total) + threads - 1) / threads;
+  if (blocks > ei_compute_units() * 16) blocks = ei_compute_units() * 16;
+  scale_cap_kernel<<<static_cast<unsigned>(blocks), threads, 0, stream>>>(
+      x, scale, cap, static_cast<size_t>(total));
   EI_LAUNCH_CHECK();
 }

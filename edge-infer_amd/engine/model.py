@@ -20,7 +20,8 @@ replace in a subclass that it registers as its `model_factory`, keeping the rest
 
 (a cap on the logits overrides `logits`, a model without a final norm `final_hidden`).  Two
 variations are options of the spec and need no subclass: `embedding_scale` multiplies the
-embedding rows, and `loop` (`config.specs.LoopSpec`) runs a span of layers several times, each
+embedding rows, `embedding_norm` norms them, `logit_scale` and `logit_softcap` scale and cap
+the logits, and `loop` (`config.specs.LoopSpec`) runs a span of layers several times, each
 pass with caches of its own, the stream being made anew before every pass from itself and the
 embedding output by a matrix [hidden, 2 hidden] and a vector per pass.  A subclass whose methods launch anything that a HIP graph
 cannot hold says so with `seams_capture_safe = False`; decode then runs eagerly.
@@ -58,6 +59,10 @@ def model_parameters(spec: ModelSpec) -> Dict[str, ParamSpec]:
     final_cls = lookup("norm", spec.final_norm.kind)
     for name, param in final_cls.parameters(spec.final_norm, spec.hidden_size).items():
         params[f"final_norm.{name}"] = param
+    if spec.embedding_norm is not None:
+        embed_cls = lookup("norm", spec.embedding_norm.kind)
+        for name, param in embed_cls.parameters(spec.embedding_norm, spec.hidden_size).items():
+            params[f"embed_norm.{name}"] = param
     params["head.weight"] = ParamSpec((spec.vocab_size, spec.hidden_size))
     params["head.bias"] = ParamSpec((spec.vocab_size,), optional=True)
     if spec.loop is not None:
@@ -155,6 +160,14 @@ class DecoderModel:
                                bias=params.get("head.bias"))
         else:  # tied: the head is the embedding table itself (no copy: same type and device)
             self.head = Linear(self.embed, self.dtype, self.device, bias=params.get("head.bias"))
+        self.embed_norm = None
+        if spec.embedding_norm is not None:
+            # a plain RMS norm on the float32 stream itself
+            if spec.embedding_norm.kind != "rmsnorm":
+                raise ValueError("the norm on the embedding rows must be of kind 'rmsnorm'")
+            self.embed_norm = lookup("norm", "rmsnorm")(
+                spec.embedding_norm, spec.hidden_size, {"weight": params["embed_norm.weight"]},
+                self.dtype, self.device)
         self.loop_in = self.loop_step = None
         self._pass_starts = {}
         if spec.loop is not None:
@@ -298,6 +311,8 @@ class DecoderModel:
         residual stream [rows, hidden]."""
         residual = ctx.buffer("residual", (ctx.n_rows, self.spec.hidden_size), torch.float32)
         lib.embed_gather(ctx.meta.tokens, self.embed, residual, self.spec.embedding_scale)
+        if self.embed_norm is not None:
+            lib.norm_rows(residual, self.embed_norm.weight, self.embed_norm.eps)
         return residual
 
     def run_layers(self, ctx, residual):
@@ -338,5 +353,9 @@ class DecoderModel:
                                         rows=ctx.meta.want_rows, write_residual=False)
 
     def logits(self, ctx, hidden) -> torch.Tensor:
-        """float32 [wanted rows, vocab] in the buffer "logits"."""
-        return self.head.forward_f32(ctx, hidden, "logits")
+        """float32 [wanted rows, vocab] in the buffer "logits": the head's products, times
+        `logit_scale`, capped by `logit_softcap` where the spec names one."""
+        logits = self.head.forward_f32(ctx, hidden, "logits")
+        if self.spec.logit_scale != 1.0 or self.spec.logit_softcap is not None:
+            lib.scale_cap(logits, self.spec.logit_scale, self.spec.logit_softcap)
+        return logits

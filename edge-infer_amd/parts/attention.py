@@ -21,6 +21,13 @@ the score of mixed queries: with the heads g of kv head c sharing the key k_c,
 sum_g T[h, g] (q_g . k_c(g)) = sum_c (sum_{g in c} T[h, g] q_g) . k_c, so the queries are mixed
 once a row (`lib.mix_heads`: a row of n_kv_heads * head_dim a head) and the generic kernel
 meets them with the keys of all kv heads laid end to end (`key_heads`).
+
+A rotation whose angles the store kernel works out itself (position kind "rope_half":
+frequencies that may be rescaled, any rotated width, values of their own width),
+`value_mix` (what a layer caches is (1 - lambda) v + lambda v_source, v_source the values that
+the step's source layer computed for the same token, kept in float32 for the step) and
+`output_gate` (the concatenated heads times sigmoid(W_g x), the gate's rows fused into the
+q/k/v product) go through `lib.head_store`, the store kernel for rows that go on after v.
 """
 from __future__ import annotations
 
@@ -51,6 +58,7 @@ TILE_US_128, MERGE_US, MERGE_SLICE_US = 1.9, 4.5, 0.1
 WAVES_A_UNIT = 16       # waves of this kernel that a compute unit holds at once
 MAX_SLICES = 32
 MAX_LAUNCH_PLANS = 512  # decode launch shapes a part remembers
+VALUE_SOURCE = "attn.v_source"   # ctx.notes / buffer: the source layer's values of this step
 
 
 @functools.lru_cache(maxsize=512)
@@ -102,6 +110,12 @@ class Attention:
                                                 init="norm")
         if spec.sink:
             params["sink"] = ParamSpec((spec.n_heads,), init="uniform", low=-1.0, high=1.0)
+        if spec.value_mix is not None:
+            # one number; the source layer and a layer that mixes nothing may hold it unused
+            params["value_mix"] = ParamSpec((), init="uniform", low=0.1, high=0.6,
+                                            optional=spec.value_mix != "mix")
+        if spec.output_gate:
+            params["gate_proj.weight"] = ParamSpec((spec.out_width, hidden))
         return params
 
     @classmethod
@@ -133,13 +147,32 @@ class Attention:
                                                  spec.head_dim, spec.v_dim))
 
     @classmethod
+    def general_store(cls, spec) -> bool:
+        """Whether the part norms, rotates and stores through `lib.head_store`."""
+        return (spec.position.kind == "rope_half" or spec.value_mix in ("source", "mix")
+                or spec.output_gate)
+
+    @classmethod
     def check(cls, spec):
         if spec.n_heads % spec.n_kv_heads:
             raise ValueError("attention: n_heads must be a multiple of n_kv_heads")
         if spec.qk_norm_scope not in ("head", "projection"):
             raise ValueError(f"attention: unknown qk_norm_scope '{spec.qk_norm_scope}'")
         whole = spec.qk_norm_scope == "projection" or not spec.qk_norm
-        if whole and spec.position.kind == "none":
+        if spec.value_mix not in (None, "off", "source", "mix"):
+            raise ValueError(f"attention: unknown value_mix '{spec.value_mix}'")
+        if cls.general_store(spec):
+            if spec.position.kind not in ("rope_half", "none"):
+                raise ValueError("attention: value mixing and the output gate are implemented "
+                                 "with position kinds 'rope_half' and 'none'")
+            if spec.qk_norm and spec.qk_norm_scope != "head":
+                raise ValueError("attention: this store norms per head only")
+            if spec.talking_heads or spec.qkv_bias:
+                raise ValueError("attention: this store takes no biases and no mixed scores")
+            if not (1 <= spec.head_dim <= 256 and 1 <= spec.v_dim <= 256):
+                raise ValueError("attention: key and value head sizes must lie in 1..256, got "
+                                 f"{spec.head_dim} and {spec.v_dim}")
+        elif whole and spec.position.kind == "none":
             # the store kernel without a rotation takes any sizes the attention kernel takes
             if not (1 <= spec.head_dim <= 256 and 1 <= spec.v_dim <= 256):
                 raise ValueError("attention: key and value head sizes must lie in 1..256, got "
@@ -173,7 +206,8 @@ class Attention:
         self.hidden = hidden
         self.dtype = dtype
         fused = torch.cat([params["q_proj.weight"], params["k_proj.weight"],
-                           params["v_proj.weight"]], dim=0)
+                           params["v_proj.weight"]]
+                          + ([params["gate_proj.weight"]] if spec.output_gate else []), dim=0)
         names = ("q_proj", "k_proj", "v_proj")
         fused_bias = None
         if any(f"{name}.bias" in params for name in names):   # absent ones count as zero
@@ -191,8 +225,13 @@ class Attention:
         self.group = spec.n_heads // spec.n_kv_heads
         self.scale = spec.scale if spec.scale is not None else spec.head_dim ** -0.5
         # without a rotation and without per-head norms, one kernel norms (or not) and stores
-        self.whole_store = (spec.position.kind == "none"
+        self.general = self.general_store(spec)
+        self.whole_store = (not self.general and spec.position.kind == "none"
                             and (spec.qk_norm_scope == "projection" or not spec.qk_norm))
+        self.value_lambda = None
+        if spec.value_mix == "mix":
+            self.value_lambda = params["value_mix"].to(device=device, dtype=torch.float32).reshape(1).contiguous()
+        self.gate_column = spec.q_width + spec.kv_width + spec.v_width    # where the gate's columns begin
         self.slopes = self.sinks = None
         if spec.distance_slope_range is not None:
             exponent = -float(spec.distance_slope_range) * torch.arange(
@@ -355,7 +394,27 @@ class Attention:
         # (the kernel that norms and stores the whole projection adds its bias as well)
         qkv, bias = (self.qkv.forward(ctx, x, "attn.qkv", bias_later=True) if self.whole_store
                      else (self.qkv.forward(ctx, x, "attn.qkv"), None))
-        if (ctx.decode and self.matrix_cores and FUSED_DECODE and qkv.dim() == 3
+        if self.general:
+            q = ctx.buffer("attn.q", (n, spec.q_width))
+            v_first, v_mode = None, 0
+            if spec.value_mix == "source":
+                # this layer's values, kept in float32 for the layers of the step that mix them in
+                v_first = ctx.buffer(VALUE_SOURCE, (n, spec.v_width), torch.float32)
+                ctx.notes[VALUE_SOURCE] = v_first
+                v_mode = 1
+            elif spec.value_mix == "mix":
+                v_first = ctx.notes.get(VALUE_SOURCE)
+                if v_first is None or tuple(v_first.shape) != (n, spec.v_width):
+                    raise ValueError("attention: a layer mixes values in, but no earlier layer of "
+                                     "the step has kept values of that width")
+                v_mode = 2
+            lib.head_store(qkv, self.q_norm, self.k_norm, spec.qk_norm_eps,
+                           getattr(self.position, "frequencies", None), meta.row_pos,
+                           meta.row_seq, page_table, q, k_pages, v_pages, spec.n_heads,
+                           spec.n_kv_heads, spec.head_dim, spec.v_dim,
+                           write_cache=entry.writes_cache, v_first=v_first, v_mode=v_mode,
+                           v_lambda=self.value_lambda)
+        elif (ctx.decode and self.matrix_cores and FUSED_DECODE and qkv.dim() == 3
                 and qkv.dtype == torch.float32 and not self.whole_store and not self.has_extras):
             # the decode kernel norms, rotates and stores for its rows itself: one launch less
             q = lib.DecodeProjection(qkv, self.q_norm, self.k_norm, spec.qk_norm_eps,
@@ -438,6 +497,8 @@ class Attention:
                               meta.row_pos, meta.row_seq, page_table, out, spec.n_heads,
                               spec.n_kv_heads, spec.head_dim, window=spec.window,
                               scale=self.scale, **more)
+        if spec.output_gate:
+            lib.gate_rows(qkv, self.gate_column, out)
         ctx.release(qkv, None if isinstance(q, lib.DecodeProjection) else q, part_o, part_ml)
         delta = self.o.forward(ctx, out, "attn.o", bias_later=bias_later)
         ctx.release(out)

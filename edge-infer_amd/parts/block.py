@@ -12,27 +12,40 @@ class PreNormBlock:
     """x += mixer(norm1(x)); x += feed_forward(norm2(x)).
     runtime/include/execution/decoder.hpp:119-168 of the reference.  The second
     addition is left pending: the next block's first norm (or the model's final
-    norm) performs it while reading the row."""
+    norm) performs it while reading the row.  A layer may have no feed-forward (then it has
+    no second norm either, and the mixer's output is what is left pending)."""
 
     parts = ("norm1", "mixer", "norm2", "ffn")
     capture_safe = True      # nothing of its own besides its parts' kernels
 
     def members(self):
         """The parts this block is made of, in the order in which they run."""
-        return (self.norm1, self.mixer, self.norm2, self.ffn)
+        return tuple(part for part in (self.norm1, self.mixer, self.norm2, self.ffn)
+                     if part is not None)
+
+    @classmethod
+    def _owners(cls, layer_spec):
+        norm_cls = lookup("norm", layer_spec.norm.kind)
+        owners = [("norm1", norm_cls, layer_spec.norm),
+                  ("mixer", lookup("mixer", layer_spec.mixer.kind), layer_spec.mixer)]
+        if layer_spec.feed_forward is not None:
+            owners += [("norm2", norm_cls, layer_spec.norm),
+                       ("ffn", lookup("feed_forward", layer_spec.feed_forward.kind),
+                        layer_spec.feed_forward)]
+        return owners
 
     @classmethod
     def parameters(cls, layer_spec, hidden):
-        norm_cls = lookup("norm", layer_spec.norm.kind)
-        mixer_cls = lookup("mixer", layer_spec.mixer.kind)
-        ffn_cls = lookup("feed_forward", layer_spec.feed_forward.kind)
         params = {}
-        for prefix, owner, spec in (("norm1", norm_cls, layer_spec.norm),
-                                    ("mixer", mixer_cls, layer_spec.mixer),
-                                    ("norm2", norm_cls, layer_spec.norm),
-                                    ("ffn", ffn_cls, layer_spec.feed_forward)):
+        for prefix, owner, spec in cls._owners(layer_spec):
             for name, param in owner.parameters(spec, hidden).items():
                 params[f"{prefix}.{name}"] = param
+        if layer_spec.feed_forward is None:
+            # a checkpoint may still hold the second norm of a layer without a feed-forward;
+            # it is taken and has no use
+            norm_cls = lookup("norm", layer_spec.norm.kind)
+            for name, param in norm_cls.parameters(layer_spec.norm, hidden).items():
+                params[f"norm2.{name}"] = ParamSpec(param.shape, init=param.init, optional=True)
         return params
 
     @classmethod
@@ -43,9 +56,8 @@ class PreNormBlock:
     def kernel_libraries(cls, layer_spec, dtype):
         """The kernel libraries its parts say they run (a part without the method says none)."""
         names = []
-        for category, spec in (("norm", layer_spec.norm), ("mixer", layer_spec.mixer),
-                               ("feed_forward", layer_spec.feed_forward)):
-            ask = getattr(lookup(category, spec.kind), "kernel_libraries", None)
+        for _, owner, spec in cls._owners(layer_spec):
+            ask = getattr(owner, "kernel_libraries", None)
             if ask is not None:
                 names.extend(ask(spec, dtype))
         return tuple(names)
@@ -56,18 +68,22 @@ class PreNormBlock:
                     if name.startswith(prefix + ".")}
         norm_cls = lookup("norm", layer_spec.norm.kind)
         mixer_cls = lookup("mixer", layer_spec.mixer.kind)
-        ffn_cls = lookup("feed_forward", layer_spec.feed_forward.kind)
         self.norm1 = norm_cls(layer_spec.norm, hidden, sub("norm1"), dtype, device)
         self.mixer = mixer_cls(layer_spec.mixer, hidden, sub("mixer"), dtype, device,
                                positions=positions)
-        self.norm2 = norm_cls(layer_spec.norm, hidden, sub("norm2"), dtype, device)
-        self.ffn = ffn_cls(layer_spec.feed_forward, hidden, sub("ffn"), dtype, device)
+        self.norm2 = self.ffn = None
+        if layer_spec.feed_forward is not None:
+            ffn_cls = lookup("feed_forward", layer_spec.feed_forward.kind)
+            self.norm2 = norm_cls(layer_spec.norm, hidden, sub("norm2"), dtype, device)
+            self.ffn = ffn_cls(layer_spec.feed_forward, hidden, sub("ffn"), dtype, device)
 
     def forward(self, ctx, residual, pending, entry):
         h = self.norm1.add_norm(ctx, residual, pending, "block.h")
         ctx.release(pending)             # added into the residual: its storage is free
         a = self.mixer.forward(ctx, h, entry)
         ctx.release(h)
+        if self.ffn is None:
+            return a
         h2 = self.norm2.add_norm(ctx, residual, a, "block.h")
         ctx.release(a)
         out = self.ffn.forward(ctx, h2)

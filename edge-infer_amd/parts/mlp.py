@@ -1,5 +1,6 @@
 """Feed-forward parts.  `GatedMLP`: down(act(gate(x)) * up(x)) with act silu or the tanh form
-of gelu; `DenseMLP`:
+of gelu, or the clamped swish: with g = min(gate(x), limit) and u = clamp(up(x), -limit, limit),
+down(g sigmoid(alpha g) (u + 1)); `DenseMLP`:
 down(act(up(x))) with act one of relu squared, relu, silu, tanh-gelu.
 
 The gated one:
@@ -92,7 +93,8 @@ class GatedMLP:
             # (the activation kernel adds the bias itself where the product left it to it)
             gate_up, bias = self.gate_up.forward(ctx, x, "mlp.gate_up", bias_later=True)
             act = ctx.buffer("mlp.act", (n, self.spec.intermediate_size))
-            lib.swiglu(gate_up, act, self.strip, self.spec.activation, bias=bias)
+            lib.swiglu(gate_up, act, self.strip, self.spec.activation, bias=bias,
+                       limit=getattr(self.spec, "limit", 0.0), alpha=getattr(self.spec, "alpha", 1.0))
             ctx.release(gate_up)
         out = self.down.forward(ctx, act, "mlp.down", bias_later=bias_later)
         ctx.release(act)

@@ -1,0 +1,69 @@
+"""Routed feed-forward: a mixture of experts.
+
+For every row x: router logits z = W_router x in float32 (the router matrix is kept in
+float32; x is read as the step stores it), the `top` experts with the largest logits, their
+weights p = softmax over the chosen logits alone, and
+
+    y = sum over the chosen e of p_e W_down,e (silu(W_gate,e x) * (W_up,e x)).
+
+The experts' matrices are stacked when the part is built (gate and up [E, F, H], down
+[E, H, F]); routing stays on the device, so a step with this part is captured like any
+other.  Kernels: `csrc/moe.hip`.
+"""
+from __future__ import annotations
+
+import torch
+
+from ..csrc import lib
+from ..weights.loader import ParamSpec
+
+
+class RoutedMLP:
+    capture_safe = True      # only this library's kernels, nothing read back, no allocation
+
+    @classmethod
+    def kernel_libraries(cls, spec, dtype):
+        return ("moe", "rowwise")
+
+    @classmethod
+    def parameters(cls, spec, hidden):
+        params = {"router.weight": ParamSpec((spec.n_experts, hidden), scale=0.2)}
+        for expert in range(spec.n_experts):
+            prefix = f"experts.{expert}."
+            params[prefix + "gate_proj.weight"] = ParamSpec((spec.intermediate_size, hidden))
+            params[prefix + "up_proj.weight"] = ParamSpec((spec.intermediate_size, hidden))
+            params[prefix + "down_proj.weight"] = ParamSpec((hidden, spec.intermediate_size))
+        return params
+
+    @classmethod
+    def check(cls, spec):
+        if not 1 <= spec.n_experts <= 512:
+            raise ValueError(f"routed_mlp: 1 to 512 experts, got {spec.n_experts}")
+        if not 1 <= spec.top <= min(spec.n_experts, 64):
+            raise ValueError(f"routed_mlp: top must lie in 1..min(experts, 64), got {spec.top}")
+        if spec.intermediate_size < 1:
+            raise ValueError("routed_mlp: an expert's width must be positive")
+
+    def __init__(self, spec, hidden, params, dtype, device):
+        self.check(spec)
+        self.spec = spec
+        self.hidden = hidden
+
+        def stacked(name):
+            return torch.stack([params[f"experts.{expert}.{name}.weight"]
+                                for expert in range(spec.n_experts)]).to(
+                                    device=device, dtype=dtype).contiguous()
+        self.w_gate, self.w_up, self.w_down = stacked("gate_proj"), stacked("up_proj"), stacked("down_proj")
+        self.router = params["router.weight"].to(device=device, dtype=torch.float32).contiguous()
+
+    def forward(self, ctx, x):
+        spec = self.spec
+        n = x.shape[0]
+        expert = ctx.buffer("moe.expert", (n, spec.top), torch.int32)
+        weight = ctx.buffer("moe.weight", (n, spec.top), torch.float32)
+        lib.moe_route(x, self.router, ctx.meta.row_seq, expert, weight)
+        act = ctx.buffer("moe.act", (n * spec.top, spec.intermediate_size))
+        out = ctx.buffer("moe.out", (n, self.hidden), torch.float32)
+        lib.moe_experts(x, self.w_gate, self.w_up, self.w_down, expert, weight, act, out)
+        ctx.release(expert, weight, act)
+        return out

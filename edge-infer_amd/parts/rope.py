@@ -11,6 +11,8 @@ the float32 angle and rounded once.  Row p holds cos for the d/2 pairs, then sin
 """
 from __future__ import annotations
 
+import math
+
 import torch
 
 
@@ -53,5 +55,35 @@ class RotaryFrequencies:
         exponent = -2.0 * torch.arange(spec.dim // 2, dtype=torch.float64) / float(spec.dim)
         frequencies = torch.pow(torch.tensor(float(spec.theta), dtype=torch.float64), exponent)
         self.frequencies = frequencies.to(torch.float32).to(device).contiguous()
+        self.table = None
+        self.max_positions = None
+
+
+def scaled_frequencies(spec) -> torch.Tensor:
+    """theta^(-2i / dim) for i < dim / 2 in float64, with the long wavelengths stretched as
+    `spec.scaling` says (see `config.specs.FrequencyScaling`)."""
+    exponent = -2.0 * torch.arange(spec.dim // 2, dtype=torch.float64) / float(spec.dim)
+    frequencies = torch.pow(torch.tensor(float(spec.theta), dtype=torch.float64), exponent)
+    scaling = getattr(spec, "scaling", None)
+    if scaling is None:
+        return frequencies
+    wavelength = 2.0 * math.pi / frequencies
+    blend = (scaling.original / wavelength - scaling.low) / (scaling.high - scaling.low)
+    between = (1.0 - blend) * frequencies / scaling.factor + blend * frequencies
+    return torch.where(wavelength < scaling.original / scaling.high, frequencies,
+                       torch.where(wavelength > scaling.original / scaling.low,
+                                   frequencies / scaling.factor, between))
+
+
+class RotaryHalfFrequencies:
+    """Rotation of the pairs (i, i + dim/2) of a head's first `dim` elements by the angle
+    position * f_i: the store kernel multiplies the float32 position by the float32 frequency
+    and takes cosine and sine itself, so there is no table and no position that is too far.
+    The frequencies are worked out in float64 (stretched where the spec says) and rounded once."""
+    def __init__(self, spec, device):
+        if spec.dim % 2 or spec.dim < 2:
+            raise ValueError("rotary dimension must be even and at least 2")
+        self.spec = spec
+        self.frequencies = scaled_frequencies(spec).to(torch.float32).to(device).contiguous()
         self.table = None
         self.max_positions = None
