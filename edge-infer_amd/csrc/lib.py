@@ -907,8 +907,8 @@ def head_store(proj, q_norm_w, k_norm_w, eps, frequencies, row_pos, row_seq, pag
                v_first=None, v_mode=0, v_lambda=None) -> None:
     """Rows that begin with [q | k | v] (and may go on with other columns), as [n, g] or float32
     slices [s, n, g]: per-head RMS norm of queries and keys (weights [head_dim], or None), the
-    rotation of every head's first R elements in pairs (i, i + R/2) by float(position) *
-    frequencies[i] (float32 [R/2], or None for no rotation), queries to `q_out`, keys
+    rotation of every head's first R elements in pairs (i, i + R/2) by position *
+    frequencies[i] (float64 [R/2], or None for no rotation), queries to `q_out`, keys
     [*, kv heads, 64, head_dim] and values [*, kv heads, 64, value_dim] to their pages.
     v_mode 1: the values are also written to `v_first` (float32 [n, kv heads * value_dim]);
     v_mode 2: what is stored is (1 - lambda) v + lambda v_first, `v_lambda` one float32 on the
@@ -947,7 +947,7 @@ def head_store(proj, q_norm_w, k_norm_w, eps, frequencies, row_pos, row_seq, pag
         _gpu(proj, "proj"), _code(proj, "proj"), nsplit, split_stride, stride,
         None if q_norm_w is None else _gpu(q_norm_w, "q_norm", torch.float32),
         None if k_norm_w is None else _gpu(k_norm_w, "k_norm", torch.float32), float(eps),
-        None if frequencies is None else _gpu(frequencies, "frequencies", torch.float32), rot_dim,
+        None if frequencies is None else _gpu(frequencies, "frequencies", torch.float64), rot_dim,
         _gpu(row_pos, "row_pos", torch.int32), _gpu(row_seq, "row_seq", torch.int32),
         _gpu(page_table, "page_table", torch.int32), page_table.shape[-1], _gpu(q_out, "q_out"),
         _gpu(k_pages, "k_pages") if write_cache else None,

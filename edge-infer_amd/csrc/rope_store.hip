@@ -616,8 +616,9 @@ extern "C" int ei_projection_norm_store(
 
 // ---------------------------------------------------------------------------------------
 // The store for heads whose values have a width of their own, whose rotation works out its
-// angles from frequencies (angle = float(position) * f_i in float32, cosine and sine taken
-// here: no table, no longest position), and whose values may be mixed with the values that
+// angles from frequencies (angle = position * f_i as a float64 product, taken modulo 2 pi and
+// rounded to float32 once, cosine and sine taken here: no table, no longest position, and the
+// float32 angle is the nearest one at any position), and whose values may be mixed with the values that
 // an earlier layer of the same step computed for the same token.
 //
 // proj: rows `row_stride` wide that begin with [q: nq * D | k: nkv * D | v: nkv * DV]
@@ -641,7 +642,7 @@ template <typename TI, typename TO>
 __global__ void head_store_kernel(
     const TI* __restrict__ proj, int nsplit, size_t split_stride, size_t row_stride,
     const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w, float eps,
-    const float* __restrict__ freqs, int R, const int32_t* __restrict__ row_pos,
+    const double* __restrict__ freqs, int R, const int32_t* __restrict__ row_pos,
     const int32_t* __restrict__ row_seq, const int32_t* __restrict__ page_table, int table_width,
     TO* __restrict__ q_out, TO* __restrict__ k_pages, TO* __restrict__ v_pages,
     float* __restrict__ v_first, int v_mode, const float* __restrict__ v_lambda,
@@ -705,7 +706,9 @@ __global__ void head_store_kernel(
     if (e < R) {
       const int partner = e < rhalf ? e + rhalf : e - rhalf;
       const float p = w ? (y[j] * inv) * w[partner] : y[j];
-      const float angle = static_cast<float>(pos) * freqs[e < rhalf ? e : e - rhalf];
+      const double turns = static_cast<double>(pos) * freqs[e < rhalf ? e : e - rhalf] *
+                           0.15915494309189535;       // in units of 2 pi
+      const float angle = static_cast<float>((turns - floor(turns)) * 6.283185307179586);
       float sn, cs;
       sincosf(angle, &sn, &cs);
       v = e < rhalf ? v * cs - p * sn : v * cs + p * sn;
@@ -718,7 +721,7 @@ __global__ void head_store_kernel(
 
 extern "C" int ei_head_store(
     const void* proj, int in_dtype, int nsplit, long long split_stride, long long row_stride,
-    const float* q_norm_w, const float* k_norm_w, float eps, const float* freqs, int rot_dim,
+    const float* q_norm_w, const float* k_norm_w, float eps, const double* freqs, int rot_dim,
     const int32_t* row_pos, const int32_t* row_seq, const int32_t* page_table, int table_width,
     void* q_out, void* k_pages, void* v_pages, int out_dtype, float* v_first, int v_mode,
     const float* v_lambda, int N, int nq, int nkv, int D, int DV, int write_cache,

@@ -77,13 +77,15 @@ def scaled_frequencies(spec) -> torch.Tensor:
 
 class RotaryHalfFrequencies:
     """Rotation of the pairs (i, i + dim/2) of a head's first `dim` elements by the angle
-    position * f_i: the store kernel multiplies the float32 position by the float32 frequency
-    and takes cosine and sine itself, so there is no table and no position that is too far.
-    The frequencies are worked out in float64 (stretched where the spec says) and rounded once."""
+    position * f_i: the store kernel multiplies the position by the float64 frequency, takes
+    the product modulo 2 pi, rounds it to float32 and takes cosine and sine itself, so there is
+    no table, no position that is too far, and the float32 angle is the nearest one however
+    far the position.  The frequencies are worked out in float64 (stretched where the spec
+    says)."""
     def __init__(self, spec, device):
         if spec.dim % 2 or spec.dim < 2:
             raise ValueError("rotary dimension must be even and at least 2")
         self.spec = spec
-        self.frequencies = scaled_frequencies(spec).to(torch.float32).to(device).contiguous()
+        self.frequencies = scaled_frequencies(spec).to(device).contiguous()
         self.table = None
         self.max_positions = None

@@ -198,13 +198,17 @@ def clamped_feed_forward(h, tensors, prefix, limit):
     return linear(g * sigmoid(1.702 * g) * (u + 1.0), tensors[prefix + "down"])
 
 
-def routed_feed_forward(h, tensors, prefix, experts, top, route_rows=None):
+def routed_feed_forward(h, tensors, prefix, experts, top, margins=None):
     """Every token runs its `top` experts with the largest router logits, weighted by the
-    softmax over those logits alone.  `route_rows` (optional): the rows the router reads, if
-    they are to differ from the experts' (a rounding of h)."""
-    logits = linear(h if route_rows is None else route_rows, tensors[prefix + "router"])
+    softmax over those logits alone.  `margins` (optional, a list) receives, per token, the gap
+    between the smallest chosen logit and the largest one that was not chosen."""
+    logits = linear(h, tensors[prefix + "router"])
     T = h.shape[0]
     out = torch.zeros(T, tensors[prefix + "e0.down"].shape[0], dtype=F64)
+    if margins is not None:
+        ordered = torch.sort(logits, dim=1, descending=True).values
+        margins.append(ordered[:, top - 1] - ordered[:, top] if top < experts
+                       else torch.full((T,), float("inf"), dtype=F64))
     for t in range(T):
         chosen = torch.topk(logits[t], top).indices
         weights = torch.softmax(logits[t][chosen], dim=0)
@@ -216,17 +220,19 @@ def routed_feed_forward(h, tensors, prefix, experts, top, route_rows=None):
     return out
 
 
-def feed_forward(h, tensors, prefix, mlp):
+def feed_forward(h, tensors, prefix, mlp, margins=None):
     if mlp["kind"] == "dense":
         return clamped_feed_forward(h, tensors, prefix, float(mlp["limit"]))
     return routed_feed_forward(h, tensors, prefix, int(mlp["router"]["experts"]),
-                               int(mlp["router"]["top"]))
+                               int(mlp["router"]["top"]), margins)
 
 
 # ---------------------------------------------------------------------------- the model
-def forward(cfg, tensors, tokens, streams=None):
+def forward(cfg, tensors, tokens, streams=None, margins=None):
     """Logits [T, vocab] (float64) of one sequence from position 0.  `streams`: a list that
-    receives the residual stream after every layer."""
+    receives the residual stream after every layer; `margins`: a list that receives, for every
+    routed feed-forward, each token's gap between its last chosen and its first unchosen
+    router logit (a token whose gap is tiny may be routed otherwise by any rounding)."""
     eps = float(cfg["norm"]["eps"])
     tokens = torch.as_tensor(tokens, dtype=torch.long)
     T = tokens.shape[0]
@@ -249,7 +255,7 @@ def forward(cfg, tensors, tokens, streams=None):
         x = x + out
         if layer.get("mlp"):
             h = rms_norm(x, tensors[prefix + "norm2"], eps)
-            x = x + feed_forward(h, tensors, prefix + "mlp.", layer["mlp"])
+            x = x + feed_forward(h, tensors, prefix + "mlp.", layer["mlp"], margins)
         if streams is not None:
             streams.append(x.clone())
     h = rms_norm(x, tensors["final.norm"], eps)
@@ -258,3 +264,23 @@ def forward(cfg, tensors, tokens, streams=None):
     if cap:
         logits = float(cap) * torch.tanh(logits / float(cap))
     return logits
+
+
+def clear_rows(cfg, tensors, tokens, least, carry=False):
+    """(logits, mask): the logits of `forward`, and at which positions no routing decision was
+    closer than `least`; with `carry`, no decision up to and including them (a choice that a
+    rounding flips at one token also reaches the tokens after it, through the mixers, if far
+    more weakly)."""
+    margins = []
+    logits = forward(cfg, tensors, tokens, margins=margins)
+    clear = torch.ones(logits.shape[0], dtype=torch.bool)
+    for gaps in margins:
+        clear &= (torch.cummin(gaps, dim=0).values if carry else gaps) > least
+    return logits, clear
+
+
+def greedy(cfg, tensors, prompt, count):
+    sequence = list(prompt)
+    for _ in range(count):
+        sequence.append(int(forward(cfg, tensors, sequence)[-1].argmax()))
+    return sequence[len(prompt):]
