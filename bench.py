@@ -2,7 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L]
                     [--shape 8b|0.6b|32b] [--only decode|prefill|generate] [--prompt P]
-                    [--with-32b] [--peaks] [--design tirurax|zadenex [--design-shape 1k|2k|4k]]
+                    [--with-32b] [--peaks] [--design tirurax|zadenex|vafepel [--design-shape 1k|2k|4k]]
 
 Prints one JSON line.  `value` is decoded tokens per second at the given batch after
 512-token prompts (one step = one decode step of the whole batch: the model, greedy
@@ -27,7 +27,10 @@ turn, dense feed-forward of four widths) beside a Qwen3 model of the same width,
 heads and parameter count, as one JSON line.  `--design zadenex` does the same for a Zadenex
 model (matrix-memory, latent-attention and window-attention layers whose scores are mixed over
 heads, gated feed-forward, one pass of a loop over the last six layers) beside the Tirurax
-model of the same width, layers, heads and parameter count.
+model of the same width, layers, heads and parameter count.  `--design vafepel` does the same
+for a Vafepel model (state-space and window-attention layers in turn, the feed-forwards in
+turn dense and routed over 8 experts) beside the Tirurax model of the same width, layers,
+heads and parameters at work for a token.
 Synthetic token ids, seeded random weights N(0, 0.02).  Peaks are the MI355X's published
 ones: HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s; `measured_peaks` (and `--peaks` alone) say what
 a plain read kernel and a loop of matrix-core products reach on the GPU at hand, and the
@@ -406,6 +409,46 @@ def zadenex_configs(shape):
     return new, old
 
 
+def vafepel_configs(shape):
+    """(Vafepel configuration, Tirurax configuration) of equal width, layers, heads, head size
+    and feed-forward parameters at work for a token: a state-space layer (heads of 64 columns,
+    128 rows of state, 8 groups) stands where a gated-delta layer stands, window attention with
+    a rotation of half the head, a sink, mixed values and an output gate where chunked
+    attention stands; the feed-forwards are in turn the dense gated one and 8 experts of half
+    its width of which a token takes 2."""
+    from edge_infer_amd.config import TiruraxConfig, VafepelConfig
+    layers, width, d_heads, d_kv, a_heads, a_kv, dim, chunk, vocab = DESIGN_SHAPES[shape]
+    ff = 4 * width
+    gated = (2 * ff // 3 + 255) // 256 * 256
+    dense = {"kind": "dense", "ff": gated, "limit": 7.0}
+    routed = {"kind": "moe", "expert": {"ff": gated // 2}, "router": {"experts": 8, "top": 2}}
+    space = {"type": "mamba2", "mixer": {"heads": width // 64, "vdim": 64, "state": 128,
+                                         "groups": 8, "conv": 4, "norm_groups": 8}}
+    window = {"type": "attention",
+              "mixer": {"heads": a_heads, "kv_heads": a_kv, "dim": dim, "vdim": dim,
+                        "scale": dim ** -0.5, "mask": {"size": chunk}, "v_mix": True,
+                        "rot": {"base": 500000.0, "dims": dim // 2,
+                                "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0,
+                                            "original": 8192}}}}
+    order = [dict(space if i % 2 == 0 else window, mlp=dense if i % 4 < 2 else routed)
+             for i in range(layers)]
+    new = VafepelConfig.from_dict({"architecture": "Vafepel", "vocab": vocab, "width": width,
+                                   "norm": {"eps": 1e-6}, "logit_scale": 1.0,
+                                   "logit_softcap": 30.0, "layers": order})
+    delta = {"type": "delta", "mixer": {"heads": d_heads, "kv_heads": d_kv, "dim": dim,
+                                        "vdim": dim, "conv": 4},
+             "mlp": {"kind": "dense", "ff": ff}}
+    attention = {"type": "attention", "mixer": {"heads": a_heads, "kv_heads": a_kv, "dim": dim,
+                                                "vdim": dim, "scale": dim ** -0.5,
+                                                "mask": {"size": chunk}},
+                 "mlp": {"kind": "dense", "ff": ff}}
+    old = TiruraxConfig.from_dict({"architecture": "Tirurax", "vocab": vocab, "width": width,
+                                   "norm": {"eps": 1e-6},
+                                   "layers": [delta if i % 2 == 0 else attention
+                                              for i in range(layers)]})
+    return new, old
+
+
 def measure_prompts(model, vocab, batch, tokens, repeats=3):
     """Best ms of one step over `batch` prompts of `tokens` tokens that start together."""
     import types
@@ -431,13 +474,16 @@ def measure_prompts(model, vocab, batch, tokens, repeats=3):
 
 def design_comparison(args):
     """Prefill and decode of the design's shape and of the closest other model of equal size
-    (Tirurax beside Qwen3, Zadenex beside Tirurax)."""
+    (Tirurax beside Qwen3, Zadenex and Vafepel beside Tirurax)."""
     import types
     import torch
     import edge_infer_amd as ei
     if args.design == "zadenex":
         new, old = zadenex_configs(args.design_shape)
         which = {"zadenex": new, "tirurax": old}
+    elif args.design == "vafepel":
+        new, old = vafepel_configs(args.design_shape)
+        which = {"vafepel": new, "tirurax": old}
     else:
         new, old = design_configs(args.design_shape)
         which = {"tirurax": new, "qwen3": old}
@@ -497,12 +543,12 @@ def main():
                         help="leave the 32B shape (decode at batch 1 and 16, prefill) out of `points`")
     parser.add_argument("--peaks", action="store_true",
                         help="measure the read and matrix-core yardsticks only")
-    parser.add_argument("--design", choices=["tirurax", "zadenex"], default=None,
+    parser.add_argument("--design", choices=["tirurax", "zadenex", "vafepel"], default=None,
                         help="measure this design beside the closest other model of equal size "
                              "(tirurax beside qwen3, zadenex beside tirurax) instead of the "
                              "default workload")
     parser.add_argument("--design-shape", choices=sorted(DESIGN_SHAPES), default="2k")
-    parser.add_argument("--design-only", choices=["zadenex", "tirurax", "qwen3"], default=None,
+    parser.add_argument("--design-only", choices=["vafepel", "zadenex", "tirurax", "qwen3"], default=None,
                         help="with --design: one of the two models only (for profiling)")
     args = parser.parse_args()
     if args.gpus != 1:
