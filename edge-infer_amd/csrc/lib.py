@@ -78,6 +78,10 @@ _SIGNATURES = {
                          c_int, c_int, c_void_p],
         "ei_moe_experts": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                            c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+        "ei_moe_grouped_supported": [c_int, c_int, c_int, c_int],
+        "ei_moe_experts_grouped": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                   c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                   c_int, c_int, c_int, c_int, c_int, c_void_p],
     },
     "delta_rule": {
         "ei_delta_conv": [c_void_p, c_int, c_int, c_longlong, c_int, c_void_p, c_int, c_void_p,
@@ -1422,6 +1426,46 @@ def moe_experts(x, w_gate, w_up, w_down, expert, weight, act, out) -> None:
                                 _gpu(weight, "weight", torch.float32), _gpu(act, "act"),
                                 _gpu(out, "out", torch.float32), n, width, inter, top, _stream())
     _check(lib, status, "moe_experts")
+
+
+def moe_grouped_supported(dtype, width: int, inter: int, n_experts: int) -> bool:
+    """Whether `moe_experts_grouped` takes these sizes (bfloat16, widths that are multiples of
+    the matrix cores' K-tile)."""
+    if dtype != torch.bfloat16:
+        return False
+    return bool(library("moe").ei_moe_grouped_supported(BF16, width, inter, n_experts))
+
+
+def moe_experts_grouped(x, w_gate, w_up, w_down, expert, weight, sorted_pairs, place, starts, act,
+                        sums, out) -> None:
+    """`moe_experts` as grouped matrix products on the matrix cores: the (row, choice) pairs are
+    laid out by expert on the device, every expert's pairs meet its matrices in tiles, and the
+    rows' weighted sums are taken last.  Scratch: sorted_pairs, place [n * top] and starts
+    [E + 1] int32, act [n * top, f] bfloat16, sums [n * top, w] float32."""
+    lib = library("moe")
+    n, width = x.shape
+    n_experts, inter = w_gate.shape[0], w_gate.shape[1]
+    top = expert.shape[1]
+    pairs = n * top
+    if tuple(w_gate.shape) != (n_experts, inter, width) or tuple(w_up.shape) != tuple(w_gate.shape) \
+            or tuple(w_down.shape) != (n_experts, width, inter):
+        raise KernelError("moe_experts_grouped: the stacked matrices have the wrong shapes")
+    if tuple(expert.shape) != (n, top) or tuple(weight.shape) != (n, top) \
+            or tuple(act.shape) != (pairs, inter) or tuple(sums.shape) != (pairs, width) \
+            or tuple(out.shape) != (n, width) or sorted_pairs.numel() < pairs \
+            or place.numel() < pairs or starts.numel() < n_experts + 1:
+        raise KernelError("moe_experts_grouped: shapes do not fit")
+    if not moe_grouped_supported(x.dtype, width, inter, n_experts):
+        raise KernelError("moe_experts_grouped: bfloat16 and widths that are multiples of 64 only")
+    status = lib.ei_moe_experts_grouped(
+        _gpu(x, "x", torch.bfloat16), _gpu(w_gate, "w_gate", torch.bfloat16),
+        _gpu(w_up, "w_up", torch.bfloat16), _gpu(w_down, "w_down", torch.bfloat16),
+        _gpu(expert, "expert", torch.int32), _gpu(weight, "weight", torch.float32),
+        _gpu(sorted_pairs, "sorted_pairs", torch.int32), _gpu(place, "place", torch.int32),
+        _gpu(starts, "starts", torch.int32), _gpu(act, "act", torch.bfloat16),
+        _gpu(sums, "sums", torch.float32), _gpu(out, "out", torch.float32), n, width, inter,
+        n_experts, top, _stream())
+    _check(lib, status, "moe_experts_grouped")
 
 
 # ---------------------------------------------------------------------------

@@ -16,36 +16,48 @@ namespace {
 constexpr int kMaxTop = 64;
 constexpr int kRouteMax = 8;      // experts a lane holds: up to 512 experts
 
-// A wave a row.
+// A block of four waves a row: the waves share the experts' logits out, the first wave chooses.
 template <typename TX>
-__global__ void moe_route_kernel(const TX* __restrict__ x, const float* __restrict__ w_router,
-                                 const int32_t* __restrict__ row_seq, int32_t* __restrict__ expert,
-                                 float* __restrict__ weight, int N, int W, int E, int top) {
-  const int wave_in_block = threadIdx.x / EI_WAVE, lane = threadIdx.x % EI_WAVE;
-  const int row = blockIdx.x * (blockDim.x / EI_WAVE) + wave_in_block;
-  if (row >= N) return;
+__global__ void __launch_bounds__(256)
+moe_route_kernel(const TX* __restrict__ x, const float* __restrict__ w_router,
+                 const int32_t* __restrict__ row_seq, int32_t* __restrict__ expert,
+                 float* __restrict__ weight, int N, int W, int E, int top) {
+  __shared__ float logits[kRouteMax * EI_WAVE];
+  const int wave = threadIdx.x / EI_WAVE, lane = threadIdx.x % EI_WAVE;
+  const int row = blockIdx.x;
   int32_t* e_out = expert + static_cast<size_t>(row) * top;
   float* w_out = weight + static_cast<size_t>(row) * top;
   if (row_seq && row_seq[row] < 0) {            // a padding row: no expert has anything to add
-    for (int k = lane; k < top; k += EI_WAVE) { e_out[k] = 0; w_out[k] = 0.f; }
+    for (int k = threadIdx.x; k < top; k += blockDim.x) { e_out[k] = 0; w_out[k] = 0.f; }
     return;
   }
   const TX* xr = x + static_cast<size_t>(row) * W;
-  float z[kRouteMax];
-#pragma unroll
-  for (int j = 0; j < kRouteMax; ++j) z[j] = -FLT_MAX;
-  for (int e = 0; e < E; ++e) {
+  for (int e = wave; e < E; e += 4) {
     const float* wr = w_router + static_cast<size_t>(e) * W;
     float sum = 0.f;
-    for (int i = lane; i < W; i += EI_WAVE) sum += ei::to_f32<TX>(xr[i]) * wr[i];
+    if (W % 4 == 0) {
+#pragma unroll 4
+      for (int i = lane * 4; i < W; i += EI_WAVE * 4) {
+        float xv[4], wv[4];
+        ei::Vec4<TX>::load(xr + i, xv);
+        ei::Vec4<float>::load(wr + i, wv);
+        sum += xv[0] * wv[0];
+        sum += xv[1] * wv[1];
+        sum += xv[2] * wv[2];
+        sum += xv[3] * wv[3];
+      }
+    } else {
+      for (int i = lane; i < W; i += EI_WAVE) sum += ei::to_f32<TX>(xr[i]) * wr[i];
+    }
     sum = ei::wave_sum(sum);
     if (!(sum > -FLT_MAX)) sum = -FLT_MAX;      // (a NaN chooses nothing ahead of a number)
-    if (e % EI_WAVE == lane) {
-#pragma unroll
-      for (int j = 0; j < kRouteMax; ++j)
-        if (j == e / EI_WAVE) z[j] = sum;
-    }
+    if (lane == 0) logits[e] = sum;
   }
+  __syncthreads();
+  if (wave != 0) return;
+  float z[kRouteMax];
+#pragma unroll
+  for (int j = 0; j < kRouteMax; ++j) z[j] = lane + j * EI_WAVE < E ? logits[lane + j * EI_WAVE] : -FLT_MAX;
   unsigned taken = 0;                            // bit j: this lane's expert lane + 64 j is chosen
   float total = 0.f, largest = 0.f;
   float mine = 0.f;                              // lane k keeps the k-th choice
@@ -171,6 +183,181 @@ moe_down_kernel(const T* __restrict__ act, const T* __restrict__ w_down,
     for (int q = 0; q < nc; ++q) out[static_cast<size_t>(row) * W + c0 + q] = total[q];
 }
 
+
+// ---------------------------------------------------------------------------------------
+// The experts as grouped matrix products on the matrix cores (bfloat16, K a multiple of 64).
+//
+// moe_group: the (row, choice) pairs counted and laid out by expert: `sorted` [P] holds the
+// pairs of expert 0, then those of expert 1, ...; `place` [P] is where a pair went (-1: a pair
+// of weight 0, which is left out); `starts` [E + 1] are the experts' first places.  Which place
+// a pair gets inside its expert's span depends on the order of the atomics; every pair is
+// computed for itself, so no result depends on it.
+__global__ void __launch_bounds__(1024)
+moe_group_kernel(const int32_t* __restrict__ expert, const float* __restrict__ weight,
+                 int32_t* __restrict__ sorted, int32_t* __restrict__ place,
+                 int32_t* __restrict__ starts, int P, int E) {
+  __shared__ int counts[kRouteMax * EI_WAVE], cursor[kRouteMax * EI_WAVE];
+  for (int e = threadIdx.x; e < E; e += blockDim.x) counts[e] = 0;
+  __syncthreads();
+  for (int p = threadIdx.x; p < P; p += blockDim.x)
+    if (weight[p] != 0.f) atomicAdd(&counts[expert[p]], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int at = 0;
+    for (int e = 0; e < E; ++e) {
+      starts[e] = at;
+      cursor[e] = at;
+      at += counts[e];
+    }
+    starts[E] = at;
+  }
+  __syncthreads();
+  for (int p = threadIdx.x; p < P; p += blockDim.x) {
+    int q = -1;
+    if (weight[p] != 0.f) {
+      q = atomicAdd(&cursor[expert[p]], 1);
+      sorted[q] = p;
+    }
+    place[p] = q;
+  }
+}
+
+typedef __bf16 moe_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float moe_f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kTileN = 64, kTileK = 64;
+
+// One tile of MB * 16 places of one expert against 64 rows of its matrix (GATED: of its gate
+// and of its up matrix).  GATED: the rows of `a` are gathered (row = pair / top) and
+// silu(gate) * up goes to `out_act` [P, N] at the pairs' places; else the rows of `a` are the
+// places themselves and the float32 products go to `out_sum` [P, N].  A wave owns 16 rows of
+// the matrix, which it reads from global memory straight into operand registers one K-tile
+// ahead; the places' rows travel through LDS (16-byte chunks stored at chunk ^ row % 8).
+template <int MB, bool GATED>
+__global__ void __launch_bounds__(256)
+moe_gemm_kernel(const bf16_t* __restrict__ a, const int32_t* __restrict__ sorted,
+                const int32_t* __restrict__ starts, const bf16_t* __restrict__ w1,
+                const bf16_t* __restrict__ w2, bf16_t* __restrict__ out_act,
+                float* __restrict__ out_sum, int E, int N, int K, int top) {
+  constexpr int TM = MB * 16;
+  constexpr int PER_THREAD = TM * (kTileK / 8) / 256 > 0 ? TM * (kTileK / 8) / 256 : 1;
+  __shared__ __attribute__((aligned(16))) bf16_t xs[TM * kTileK];
+  __shared__ int tile_info[2];
+  if (threadIdx.x == 0) {       // which expert's tile this block is
+    int t = blockIdx.x, found = -1, m0 = 0;
+    for (int e = 0; e < E; ++e) {
+      const int count = starts[e + 1] - starts[e];
+      const int tiles = (count + TM - 1) / TM;
+      if (t < tiles) { found = e; m0 = t * TM; break; }
+      t -= tiles;
+    }
+    tile_info[0] = found;
+    tile_info[1] = m0;
+  }
+  __syncthreads();
+  const int e = tile_info[0];
+  if (e < 0) return;
+  const int first = starts[e] + tile_info[1];                 // the tile's first place
+  const int valid = min(TM, starts[e + 1] - first);           // places of the tile that exist
+  const int wave = threadIdx.x / EI_WAVE, lane = threadIdx.x % EI_WAVE;
+  const int r16 = lane % 16, quarter = lane / 16;
+  const int n_wave = blockIdx.y * kTileN + wave * 16;         // the wave's first matrix row
+  const int n_row = min(n_wave + r16, N - 1);                 // (clamped: rows beyond N are not stored)
+  const bf16_t* w1_row = w1 + (static_cast<size_t>(e) * N + n_row) * K + quarter * 8;
+  const bf16_t* w2_row = GATED ? w2 + (static_cast<size_t>(e) * N + n_row) * K + quarter * 8 : nullptr;
+  // the chunks of the places' rows that this thread carries into LDS
+  const bf16_t* src[PER_THREAD];
+  int dst[PER_THREAD];
+#pragma unroll
+  for (int i = 0; i < PER_THREAD; ++i) {
+    const int index = threadIdx.x + i * 256;
+    const int row = index / (kTileK / 8), chunk = index % (kTileK / 8);
+    const int at = first + min(row, valid - 1);               // (clamped: such rows are not stored)
+    const size_t source_row = GATED ? static_cast<size_t>(sorted[at] / top) : static_cast<size_t>(at);
+    src[i] = a + source_row * K + chunk * 8;
+    dst[i] = row * kTileK + ((chunk ^ (row % 8)) * 8);
+  }
+  const bool carries = threadIdx.x < TM * (kTileK / 8);      // (tiles of fewer chunks than threads)
+  moe_f32x4 acc1[MB], acc2[GATED ? MB : 1];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) {
+    acc1[mb] = moe_f32x4{0.f, 0.f, 0.f, 0.f};
+    if (GATED) acc2[mb] = moe_f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  uint4 x_next[PER_THREAD];
+  moe_bf16x8 wa[2], wb[2], wa_next[2], wb_next[2];
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < PER_THREAD; ++i)
+      if (carries) x_next[i] = *reinterpret_cast<const uint4*>(src[i] + k0);
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      wa_next[s] = *reinterpret_cast<const moe_bf16x8*>(w1_row + k0 + s * 32);
+      if (GATED) wb_next[s] = *reinterpret_cast<const moe_bf16x8*>(w2_row + k0 + s * 32);
+    }
+  };
+  fetch(0);
+  for (int k0 = 0; k0 < K; k0 += kTileK) {
+    __syncthreads();                       // everybody has read the tile before
+#pragma unroll
+    for (int i = 0; i < PER_THREAD; ++i)
+      if (carries) *reinterpret_cast<uint4*>(&xs[dst[i]]) = x_next[i];
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      wa[s] = wa_next[s];
+      if (GATED) wb[s] = wb_next[s];
+    }
+    __syncthreads();
+    if (k0 + kTileK < K) fetch(k0 + kTileK);
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) {
+        const int row = mb * 16 + r16, chunk = s * 4 + quarter;
+        const moe_bf16x8 xf = *reinterpret_cast<const moe_bf16x8*>(
+            &xs[row * kTileK + ((chunk ^ (row % 8)) * 8)]);
+        acc1[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[s], xf, acc1[mb], 0, 0, 0);
+        if (GATED) acc2[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb[s], xf, acc2[mb], 0, 0, 0);
+      }
+    }
+  }
+  // lane (r16, quarter) holds, of place mb * 16 + r16, the matrix rows n_wave + 4 quarter + i
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) {
+    const int row = mb * 16 + r16;
+    if (row >= valid) continue;
+    const size_t at = static_cast<size_t>(first + row) * N;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int n = n_wave + 4 * quarter + i;
+      if (n >= N) continue;
+      if (GATED) {
+        const float gate = acc1[mb][i], up = acc2[mb][i];
+        out_act[at + n] = ei::f32_to_bf16(gate / (1.0f + expf(-gate)) * up);
+      } else {
+        out_sum[at + n] = acc1[mb][i];
+      }
+    }
+  }
+}
+
+// out [rows, W] = sum over a row's choices of weight * the choice's product row.
+__global__ void moe_combine_kernel(const float* __restrict__ sums, const int32_t* __restrict__ place,
+                                   const float* __restrict__ weight, float* __restrict__ out,
+                                   int W, int top, size_t total) {
+  const size_t start = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const size_t step = static_cast<size_t>(gridDim.x) * blockDim.x;
+  for (size_t idx = start; idx < total; idx += step) {
+    const size_t row = idx / W, col = idx % W;
+    float sum = 0.f;
+    for (int k = 0; k < top; ++k) {
+      const int q = place[row * top + k];
+      if (q >= 0) sum += weight[row * top + k] * sums[static_cast<size_t>(q) * W + col];
+    }
+    out[idx] = sum;
+  }
+}
+
 }  // namespace
 
 extern "C" int ei_moe_route(const void* x, int x_dtype, const float* w_router, const int32_t* row_seq,
@@ -180,7 +367,7 @@ extern "C" int ei_moe_route(const void* x, int x_dtype, const float* w_router, c
   EI_REQUIRE(E >= 1 && E <= kRouteMax * EI_WAVE && top >= 1 && top <= E && top <= kMaxTop,
              "moe_route: up to 512 experts, of which 1 to 64 are chosen");
   const int threads = 256;
-  const unsigned blocks = static_cast<unsigned>((N + 3) / 4);
+  const unsigned blocks = static_cast<unsigned>(N);
   if (x_dtype == EI_F32)
     moe_route_kernel<float><<<blocks, threads, 0, stream>>>(static_cast<const float*>(x), w_router,
                                                             row_seq, expert, weight, N, W, E, top);
@@ -212,5 +399,51 @@ extern "C" int ei_moe_experts(const void* x, const void* w_gate, const void* w_u
   else if (dtype == EI_BF16) EI_MOE(bf16_t);
   else EI_REQUIRE(false, "moe_experts: unknown dtype");
 #undef EI_MOE
+  EI_LAUNCH_CHECK();
+}
+
+// Whether `ei_moe_experts_grouped` takes these sizes.
+extern "C" int ei_moe_grouped_supported(int dtype, int W, int F, int E) {
+  return dtype == EI_BF16 && W % kTileK == 0 && F % kTileK == 0 && E <= kRouteMax * EI_WAVE ? 1 : 0;
+}
+
+// The experts as grouped products.  Scratch: sorted, place [P] and starts [E + 1] int32,
+// act [P, F] bfloat16, sums [P, W] float32, with P = N * top.
+extern "C" int ei_moe_experts_grouped(const void* x, const void* w_gate, const void* w_up,
+                                      const void* w_down, const int32_t* expert, const float* weight,
+                                      int32_t* sorted, int32_t* place, int32_t* starts, void* act,
+                                      float* sums, float* out, int N, int W, int F, int E, int top,
+                                      hipStream_t stream) {
+  EI_REQUIRE(x && w_gate && w_up && w_down && expert && weight && sorted && place && starts && act &&
+                 sums && out, "moe_experts_grouped: null pointer");
+  EI_REQUIRE(N > 0 && top >= 1 && E >= 1 && ei_moe_grouped_supported(EI_BF16, W, F, E),
+             "moe_experts_grouped: sizes it does not take");
+  const long long pairs = static_cast<long long>(N) * top;
+  EI_REQUIRE(pairs <= 0x3fffffffLL, "moe_experts_grouped: too many rows for one launch");
+  const int P = static_cast<int>(pairs);
+  moe_group_kernel<<<1, 1024, 0, stream>>>(expert, weight, sorted, place, starts, P, E);
+  const bf16_t* xb = static_cast<const bf16_t*>(x);
+  const bf16_t* g = static_cast<const bf16_t*>(w_gate);
+  const bf16_t* u = static_cast<const bf16_t*>(w_up);
+  const bf16_t* d = static_cast<const bf16_t*>(w_down);
+  bf16_t* ab = static_cast<bf16_t*>(act);
+  // tiles of 32 places while an expert has few (decoding), of 128 for prompts
+  if (P <= 32 * E) {
+    const unsigned tiles = static_cast<unsigned>((P + 31) / 32 + E);
+    moe_gemm_kernel<2, true><<<dim3(tiles, (F + kTileN - 1) / kTileN), 256, 0, stream>>>(
+        xb, sorted, starts, g, u, ab, nullptr, E, F, W, top);
+    moe_gemm_kernel<2, false><<<dim3(tiles, (W + kTileN - 1) / kTileN), 256, 0, stream>>>(
+        ab, sorted, starts, d, nullptr, nullptr, sums, E, W, F, top);
+  } else {
+    const unsigned tiles = static_cast<unsigned>((P + 127) / 128 + E);
+    moe_gemm_kernel<8, true><<<dim3(tiles, (F + kTileN - 1) / kTileN), 256, 0, stream>>>(
+        xb, sorted, starts, g, u, ab, nullptr, E, F, W, top);
+    moe_gemm_kernel<8, false><<<dim3(tiles, (W + kTileN - 1) / kTileN), 256, 0, stream>>>(
+        ab, sorted, starts, d, nullptr, nullptr, sums, E, W, F, top);
+  }
+  const size_t total = static_cast<size_t>(N) * W;
+  size_t blocks = (total + 255) / 256;
+  if (blocks > static_cast<size_t>(ei_compute_units()) * 16) blocks = static_cast<size_t>(ei_compute_units()) * 16;
+  moe_combine_kernel<<<static_cast<unsigned>(blocks), 256, 0, stream>>>(sums, place, weight, out, W, top, total);
   EI_LAUNCH_CHECK();
 }

@@ -82,12 +82,32 @@ __global__ void ssm_tail_kernel(const TI* __restrict__ proj, int nsplit, size_t 
   new_tail[static_cast<size_t>(j) * C + c] = x;
 }
 
+// Sum over the L neighbouring lanes (L a power of two, the group's first lane a multiple of L)
+// that share a column, every lane getting it: DPP adds inside a row of 16 lanes, row swaps
+// beyond; no step goes through LDS.
+__device__ __forceinline__ float group_sum(float v, int L) {
+  if (L >= 2) v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xb1, 0xf, 0xf, false));   // quad_perm [1,0,3,2]
+  if (L >= 4) v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4e, 0xf, 0xf, false));   // quad_perm [2,3,0,1]
+  if (L >= 8) v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xf, 0xf, false));  // row_half_mirror
+  if (L >= 16) v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xf, 0xf, false)); // row_mirror
+  if (L >= 32) {
+    const ei::ei_u32x2 r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = __uint_as_float(r.x) + __uint_as_float(r.y);
+  }
+  if (L >= 64) {
+    const ei::ei_u32x2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = __uint_as_float(r.x) + __uint_as_float(r.y);
+  }
+  return v;
+}
+
 constexpr int kScanRows = 16;     // rows of S a thread owns
 constexpr int kScanTile = 16;     // tokens staged through LDS at a time
 constexpr int kScanThreads = 256;
 
 // A block a (sequence, head, block of columns of S).  A thread owns kScanRows rows of one
-// column; the L = Npad / kScanRows lanes of a column add their partial read-outs by shuffles.
+// column; the L = Npad / kScanRows lanes of a column add their partial read-outs, a tile's
+// tokens side by side once the tile is walked, so that only S is a chain from token to token.
 template <typename TI>
 __global__ void __launch_bounds__(kScanThreads)
 ssm_scan_kernel(const float* __restrict__ conv, const TI* __restrict__ proj, int nsplit,
@@ -121,8 +141,19 @@ ssm_scan_kernel(const float* __restrict__ conv, const TI* __restrict__ proj, int
                       (static_cast<size_t>(head) * P + (live ? col : 0)) * Nst;
   float* s_out = state + static_cast<size_t>(seq_out[seq]) * state_stride +
                  (static_cast<size_t>(head) * P + (live ? col : 0)) * Nst;
+  // (rows in 16-byte pieces where the state's rows and the head's columns begin on such)
+  const bool pieces = Nst % 4 == 0 && state_stride % 4 == 0;
+  if (pieces) {
 #pragma unroll
-  for (int r = 0; r < kScanRows; ++r) S[r] = (live && n0 + r < Nst) ? s_in[n0 + r] : 0.f;
+    for (int r = 0; r < kScanRows; r += 4) {
+      const float4 v = (live && n0 + r < Nst) ? *reinterpret_cast<const float4*>(s_in + n0 + r)
+                                              : make_float4(0.f, 0.f, 0.f, 0.f);
+      S[r] = v.x; S[r + 1] = v.y; S[r + 2] = v.z; S[r + 3] = v.w;
+    }
+  } else {
+#pragma unroll
+    for (int r = 0; r < kScanRows; ++r) S[r] = (live && n0 + r < Nst) ? s_in[n0 + r] : 0.f;
+  }
   const float rate = expf(a_log[head]), bias = dt_bias[head], skip = d_skip[head];
   const int row0 = seq_row0[seq];
 
@@ -147,7 +178,11 @@ ssm_scan_kernel(const float* __restrict__ conv, const TI* __restrict__ proj, int
       decays[tid] = expf(-rate * dt);
     }
     __syncthreads();
-    for (int t = 0; t < nt; ++t) {
+    float sums[kScanTile];
+#pragma unroll
+    for (int t = 0; t < kScanTile; ++t) {
+      sums[t] = 0.f;
+      if (t >= nt) continue;
       const float dt = dts[t], decay = decays[t];
       const float x = xs[t * cols + col_local];
       const float xdt = x * dt;
@@ -167,15 +202,28 @@ ssm_scan_kernel(const float* __restrict__ conv, const TI* __restrict__ proj, int
         acc += S[r + 2] * cv.z;
         acc += S[r + 3] * cv.w;
       }
-      for (int offset = L / 2; offset > 0; offset >>= 1) acc += __shfl_xor(acc, offset, EI_WAVE);
+      sums[t] = acc;
+    }
+#pragma unroll
+    for (int t = 0; t < kScanTile; ++t) {
+      if (t >= nt) continue;
+      const float total = group_sum(sums[t], L);
       if (live && sub == 0)
-        y_raw[static_cast<size_t>(row0 + t0 + t) * inner + head * P + col] = acc + skip * x;
+        y_raw[static_cast<size_t>(row0 + t0 + t) * inner + head * P + col] =
+            total + skip * xs[t * cols + col_local];
     }
   }
   if (live) {
+    if (pieces) {
 #pragma unroll
-    for (int r = 0; r < kScanRows; ++r)
-      if (n0 + r < Nst) s_out[n0 + r] = S[r];
+      for (int r = 0; r < kScanRows; r += 4)
+        if (n0 + r < Nst)
+          *reinterpret_cast<float4*>(s_out + n0 + r) = make_float4(S[r], S[r + 1], S[r + 2], S[r + 3]);
+    } else {
+#pragma unroll
+      for (int r = 0; r < kScanRows; ++r)
+        if (n0 + r < Nst) s_out[n0 + r] = S[r];
+    }
   }
 }
 

@@ -8,7 +8,9 @@ weights p = softmax over the chosen logits alone, and
 
 The experts' matrices are stacked when the part is built (gate and up [E, F, H], down
 [E, H, F]); routing stays on the device, so a step with this part is captured like any
-other.  Kernels: `csrc/moe.hip`.
+other.  In bfloat16 with widths that are multiples of 64 the experts run as grouped matrix
+products on the matrix cores (the pairs of (row, choice) laid out by expert on the device);
+otherwise, and in float32, a kernel takes one pair at a time.  Kernels: `csrc/moe.hip`.
 """
 from __future__ import annotations
 
@@ -55,6 +57,8 @@ class RoutedMLP:
                                     device=device, dtype=dtype).contiguous()
         self.w_gate, self.w_up, self.w_down = stacked("gate_proj"), stacked("up_proj"), stacked("down_proj")
         self.router = params["router.weight"].to(device=device, dtype=torch.float32).contiguous()
+        self.grouped = lib.moe_grouped_supported(dtype, hidden, spec.intermediate_size,
+                                                 spec.n_experts)
 
     def forward(self, ctx, x):
         spec = self.spec
@@ -64,6 +68,15 @@ class RoutedMLP:
         lib.moe_route(x, self.router, ctx.meta.row_seq, expert, weight)
         act = ctx.buffer("moe.act", (n * spec.top, spec.intermediate_size))
         out = ctx.buffer("moe.out", (n, self.hidden), torch.float32)
-        lib.moe_experts(x, self.w_gate, self.w_up, self.w_down, expert, weight, act, out)
+        if self.grouped:
+            pairs = n * spec.top
+            order = ctx.buffer("moe.order", (2 * pairs + spec.n_experts + 1,), torch.int32)
+            sums = ctx.buffer("moe.sums", (pairs, self.hidden), torch.float32)
+            lib.moe_experts_grouped(x, self.w_gate, self.w_up, self.w_down, expert, weight,
+                                    order[:pairs], order[pairs:2 * pairs], order[2 * pairs:], act,
+                                    sums, out)
+            ctx.release(order, sums)
+        else:
+            lib.moe_experts(x, self.w_gate, self.w_up, self.w_down, expert, weight, act, out)
         ctx.release(expert, weight, act)
         return out

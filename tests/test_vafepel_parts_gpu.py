@@ -522,14 +522,17 @@ def test_of_equal_logits_the_lower_index_is_chosen():
     assert expert.cpu().tolist() == [[2, 4, 7, 0, 1]] * 2
 
 
-@pytest.mark.parametrize("experts, top, inter, width", [(6, 2, 40, 48), (9, 3, 13, 50), (4, 1, 96, 64)])
+@pytest.mark.parametrize("experts, top, inter, width, rows", [
+    (6, 2, 40, 48, 21), (9, 3, 13, 50, 21), (4, 1, 96, 64, 21), (5, 2, 128, 64, 3),
+    (3, 2, 192, 128, 700), (12, 3, 64, 192, 77)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_the_experts_of_a_rows_choice(experts, top, inter, width, dtype):
+def test_the_experts_of_a_rows_choice(experts, top, inter, width, rows, dtype):
     """The experts' kernels on the router kernel's own choice, against the plain expert run on
-    that choice (so that no close call of the router enters)."""
+    that choice (so that no close call of the router enters).  In bfloat16, widths that are
+    multiples of 64 take the grouped products on the matrix cores: tiles of 32 places for few
+    rows, of 128 for many, experts with no row at all, tiles that an expert fills in part."""
     from edge_infer_amd.csrc import lib
     torch.manual_seed(inter)
-    rows = 21
     x = torch.randn(rows, width).to(torch.bfloat16).float()
     router = torch.randn(experts, width)
     gate, up = (torch.randn(experts, inter, width) / width ** 0.5 for _ in range(2))
@@ -541,7 +544,17 @@ def test_the_experts_of_a_rows_choice(experts, top, inter, width, dtype):
     lib.moe_route(xd, router.to(DEV), None, expert, weight)
     act = torch.empty(rows * top, inter, device=DEV, dtype=dtype)
     out = torch.empty(rows, width, device=DEV)
-    lib.moe_experts(xd, *(t.to(DEV).to(dtype) for t in (gate, up, down)), expert, weight, act, out)
+    matrices = [t.to(DEV).to(dtype) for t in (gate, up, down)]
+    if lib.moe_grouped_supported(dtype, width, inter, experts):
+        pairs = rows * top
+        order = torch.empty(2 * pairs + experts + 1, dtype=torch.int32, device=DEV)
+        sums = torch.empty(pairs, width, device=DEV)
+        lib.moe_experts_grouped(xd, *matrices, expert, weight, order[:pairs], order[pairs:2 * pairs],
+                                order[2 * pairs:], act, sums, out)
+        assert sorted(order[:pairs].tolist()) == list(range(pairs))
+    else:
+        assert dtype == torch.float32 or width % 64 or inter % 64
+        lib.moe_experts(xd, *matrices, expert, weight, act, out)
     want = torch.zeros(rows, width, dtype=torch.float64)
     for r in range(rows):
         for k in range(top):
