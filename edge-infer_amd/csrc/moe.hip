@@ -225,23 +225,25 @@ moe_group_kernel(const int32_t* __restrict__ expert, const float* __restrict__ w
 typedef __bf16 moe_bf16x8 __attribute__((ext_vector_type(8)));
 typedef float moe_f32x4 __attribute__((ext_vector_type(4)));
 
-constexpr int kTileN = 64, kTileK = 64;
+constexpr int kTileN = 64, kTileK = 64;      // (kTileK: the least K-tile; K must be a multiple)
 
 // One tile of MB * 16 places of one expert against 64 rows of its matrix (GATED: of its gate
 // and of its up matrix).  GATED: the rows of `a` are gathered (row = pair / top) and
 // silu(gate) * up goes to `out_act` [P, N] at the pairs' places; else the rows of `a` are the
 // places themselves and the float32 products go to `out_sum` [P, N].  A wave owns 16 rows of
 // the matrix, which it reads from global memory straight into operand registers one K-tile
-// ahead; the places' rows travel through LDS (16-byte chunks stored at chunk ^ row % 8).
-template <int MB, bool GATED>
+// ahead; the places' rows travel through LDS (16-byte chunks stored at chunk ^ row % 8).  KT is
+// the K-tile: 64 for the large tiles of prompts, 256 for the small ones of decoding, where a
+// wave has little to multiply and lives on how many loads of the matrix it keeps in flight.
+template <int MB, bool GATED, int KT>
 __global__ void __launch_bounds__(256)
 moe_gemm_kernel(const bf16_t* __restrict__ a, const int32_t* __restrict__ sorted,
                 const int32_t* __restrict__ starts, const bf16_t* __restrict__ w1,
                 const bf16_t* __restrict__ w2, bf16_t* __restrict__ out_act,
                 float* __restrict__ out_sum, int E, int N, int K, int top) {
   constexpr int TM = MB * 16;
-  constexpr int PER_THREAD = TM * (kTileK / 8) / 256 > 0 ? TM * (kTileK / 8) / 256 : 1;
-  __shared__ __attribute__((aligned(16))) bf16_t xs[TM * kTileK];
+  constexpr int PER_THREAD = TM * (KT / 8) / 256 > 0 ? TM * (KT / 8) / 256 : 1;
+  __shared__ __attribute__((aligned(16))) bf16_t xs[TM * KT];
   __shared__ int tile_info[2];
   if (threadIdx.x == 0) {       // which expert's tile this block is
     int t = blockIdx.x, found = -1, m0 = 0;
@@ -271,13 +273,13 @@ moe_gemm_kernel(const bf16_t* __restrict__ a, const int32_t* __restrict__ sorted
 #pragma unroll
   for (int i = 0; i < PER_THREAD; ++i) {
     const int index = threadIdx.x + i * 256;
-    const int row = index / (kTileK / 8), chunk = index % (kTileK / 8);
+    const int row = index / (KT / 8), chunk = index % (KT / 8);
     const int at = first + min(row, valid - 1);               // (clamped: such rows are not stored)
     const size_t source_row = GATED ? static_cast<size_t>(sorted[at] / top) : static_cast<size_t>(at);
     src[i] = a + source_row * K + chunk * 8;
-    dst[i] = row * kTileK + ((chunk ^ (row % 8)) * 8);
+    dst[i] = row * KT + ((chunk ^ (row % 8)) * 8);
   }
-  const bool carries = threadIdx.x < TM * (kTileK / 8);      // (tiles of fewer chunks than threads)
+  const bool carries = threadIdx.x < TM * (KT / 8);      // (tiles of fewer chunks than threads)
   moe_f32x4 acc1[MB], acc2[GATED ? MB : 1];
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
@@ -285,37 +287,38 @@ moe_gemm_kernel(const bf16_t* __restrict__ a, const int32_t* __restrict__ sorted
     if (GATED) acc2[mb] = moe_f32x4{0.f, 0.f, 0.f, 0.f};
   }
   uint4 x_next[PER_THREAD];
-  moe_bf16x8 wa[2], wb[2], wa_next[2], wb_next[2];
+  constexpr int STEPS = KT / 32;
+  moe_bf16x8 wa[STEPS], wb[GATED ? STEPS : 1], wa_next[STEPS], wb_next[GATED ? STEPS : 1];
   auto fetch = [&](int k0) {
 #pragma unroll
     for (int i = 0; i < PER_THREAD; ++i)
       if (carries) x_next[i] = *reinterpret_cast<const uint4*>(src[i] + k0);
 #pragma unroll
-    for (int s = 0; s < 2; ++s) {
+    for (int s = 0; s < STEPS; ++s) {
       wa_next[s] = *reinterpret_cast<const moe_bf16x8*>(w1_row + k0 + s * 32);
       if (GATED) wb_next[s] = *reinterpret_cast<const moe_bf16x8*>(w2_row + k0 + s * 32);
     }
   };
   fetch(0);
-  for (int k0 = 0; k0 < K; k0 += kTileK) {
+  for (int k0 = 0; k0 < K; k0 += KT) {
     __syncthreads();                       // everybody has read the tile before
 #pragma unroll
     for (int i = 0; i < PER_THREAD; ++i)
       if (carries) *reinterpret_cast<uint4*>(&xs[dst[i]]) = x_next[i];
 #pragma unroll
-    for (int s = 0; s < 2; ++s) {
+    for (int s = 0; s < STEPS; ++s) {
       wa[s] = wa_next[s];
       if (GATED) wb[s] = wb_next[s];
     }
     __syncthreads();
-    if (k0 + kTileK < K) fetch(k0 + kTileK);
+    if (k0 + KT < K) fetch(k0 + KT);
 #pragma unroll
-    for (int s = 0; s < 2; ++s) {
+    for (int s = 0; s < STEPS; ++s) {
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
         const int row = mb * 16 + r16, chunk = s * 4 + quarter;
         const moe_bf16x8 xf = *reinterpret_cast<const moe_bf16x8*>(
-            &xs[row * kTileK + ((chunk ^ (row % 8)) * 8)]);
+            &xs[row * KT + ((chunk ^ (row % 8)) * 8)]);
         acc1[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[s], xf, acc1[mb], 0, 0, 0);
         if (GATED) acc2[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb[s], xf, acc2[mb], 0, 0, 0);
       }
@@ -430,15 +433,23 @@ extern "C" int ei_moe_experts_grouped(const void* x, const void* w_gate, const v
   // tiles of 32 places while an expert has few (decoding), of 128 for prompts
   if (P <= 32 * E) {
     const unsigned tiles = static_cast<unsigned>((P + 31) / 32 + E);
-    moe_gemm_kernel<2, true><<<dim3(tiles, (F + kTileN - 1) / kTileN), 256, 0, stream>>>(
-        xb, sorted, starts, g, u, ab, nullptr, E, F, W, top);
-    moe_gemm_kernel<2, false><<<dim3(tiles, (W + kTileN - 1) / kTileN), 256, 0, stream>>>(
-        ab, sorted, starts, d, nullptr, nullptr, sums, E, W, F, top);
+    const dim3 grid_up(tiles, (F + kTileN - 1) / kTileN), grid_down(tiles, (W + kTileN - 1) / kTileN);
+    // (the long K-tile where few experts are at work and their waves cannot fill the chip:
+    // measured at 2, 16 and 128 pairs over 8 experts of 2,816 x 2,048)
+    const bool few = P <= 4;
+    if (few && W % 256 == 0)
+      moe_gemm_kernel<2, true, 256><<<grid_up, 256, 0, stream>>>(xb, sorted, starts, g, u, ab, nullptr, E, F, W, top);
+    else
+      moe_gemm_kernel<2, true, 64><<<grid_up, 256, 0, stream>>>(xb, sorted, starts, g, u, ab, nullptr, E, F, W, top);
+    if (few && F % 256 == 0)
+      moe_gemm_kernel<2, false, 256><<<grid_down, 256, 0, stream>>>(ab, sorted, starts, d, nullptr, nullptr, sums, E, W, F, top);
+    else
+      moe_gemm_kernel<2, false, 64><<<grid_down, 256, 0, stream>>>(ab, sorted, starts, d, nullptr, nullptr, sums, E, W, F, top);
   } else {
     const unsigned tiles = static_cast<unsigned>((P + 127) / 128 + E);
-    moe_gemm_kernel<8, true><<<dim3(tiles, (F + kTileN - 1) / kTileN), 256, 0, stream>>>(
+    moe_gemm_kernel<8, true, 64><<<dim3(tiles, (F + kTileN - 1) / kTileN), 256, 0, stream>>>(
         xb, sorted, starts, g, u, ab, nullptr, E, F, W, top);
-    moe_gemm_kernel<8, false><<<dim3(tiles, (W + kTileN - 1) / kTileN), 256, 0, stream>>>(
+    moe_gemm_kernel<8, false, 64><<<dim3(tiles, (W + kTileN - 1) / kTileN), 256, 0, stream>>>(
         ab, sorted, starts, d, nullptr, nullptr, sums, E, W, F, top);
   }
   const size_t total = static_cast<size_t>(N) * W;
