@@ -5,9 +5,11 @@
 // weights softmax(z over the chosen ones only).  Experts: for row r and its choice k with expert
 // e and weight p,  y_r += p W_down,e (silu(W_gate,e x_r) * (W_up,e x_r)).
 //
-// These kernels take a row's experts one (row, choice) pair at a time and stream the expert's
-// matrices for it: the form for few rows (decoding), and a correct one for any number.  The
-// matrices of all experts lie stacked: gate and up [E, F, W], down [E, W, F].
+// Two forms of the experts.  One takes a (row, choice) pair at a time and streams the expert's
+// matrices for it: any type and any sizes.  The other (bfloat16, widths that are multiples of
+// 64) lays the pairs out by expert on the device and runs every expert's pairs against its
+// matrices as tiles on the matrix cores.  The matrices of all experts lie stacked: gate and up
+// [E, F, W], down [E, W, F].
 #include "common.h"
 #include <float.h>
 

@@ -25,16 +25,35 @@ __device__ __forceinline__ float sliced(const TI* p, int nsplit, size_t split_st
   return v;
 }
 
+template <typename TI>
+__device__ __forceinline__ void ssm_tail_element(const TI* proj, int nsplit, size_t split_stride,
+                                                 size_t row_stride, int col0, float* state,
+                                                 size_t state_stride, size_t tail_offset,
+                                                 const int32_t* seq_in, const int32_t* seq_out,
+                                                 const int32_t* seq_count, const int32_t* seq_row0,
+                                                 int n_seqs, int C, int J, size_t idx);
+
 // conv [N, C] float32 = silu(bias + sum_j w[c, j] * input(t - (J - 1) + j)); inputs before the
-// step's first row come from the sequence's tail in the state.  A thread a (row, channel).
+// step's first row come from the sequence's tail in the state.  A thread a (row, channel);
+// the threads beyond those renew the tails (a thread a (sequence, tap, channel)): the new tail
+// is written to another row of the state than the old one is read from.
 template <typename TI>
 __global__ void ssm_conv_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride,
                                 size_t row_stride, int col0, const float* __restrict__ w,
-                                const float* __restrict__ bias, const float* __restrict__ state,
+                                const float* __restrict__ bias, const float* state,
                                 size_t state_stride, size_t tail_offset,
                                 const int32_t* __restrict__ row_pos, const int32_t* __restrict__ row_seq,
                                 const int32_t* __restrict__ seq_in, const int32_t* __restrict__ seq_start,
-                                float* __restrict__ conv, int N, int C, int J) {
+                                float* __restrict__ conv, int N, int C, int J,
+                                float* state_out, const int32_t* __restrict__ seq_out,
+                                const int32_t* __restrict__ seq_count,
+                                const int32_t* __restrict__ seq_row0, int n_seqs, unsigned conv_blocks) {
+  if (blockIdx.x >= conv_blocks) {
+    ssm_tail_element(proj, nsplit, split_stride, row_stride, col0, state_out, state_stride,
+                     tail_offset, seq_in, seq_out, seq_count, seq_row0, n_seqs, C, J,
+                     static_cast<size_t>(blockIdx.x - conv_blocks) * blockDim.x + threadIdx.x);
+    return;
+  }
   const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (idx >= static_cast<size_t>(N) * C) return;
   const int row = static_cast<int>(idx / C), c = static_cast<int>(idx % C);
@@ -58,13 +77,12 @@ __global__ void ssm_conv_kernel(const TI* __restrict__ proj, int nsplit, size_t 
 // The new tail of every sequence: its last J - 1 inputs, from the step's rows or, where the
 // step brought fewer, from the old tail.  A thread a (sequence, tap, channel).
 template <typename TI>
-__global__ void ssm_tail_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride,
-                                size_t row_stride, int col0, float* __restrict__ state,
-                                size_t state_stride, size_t tail_offset,
-                                const int32_t* __restrict__ seq_in, const int32_t* __restrict__ seq_out,
-                                const int32_t* __restrict__ seq_count, const int32_t* __restrict__ seq_row0,
-                                int n_seqs, int C, int J) {
-  const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+__device__ __forceinline__ void ssm_tail_element(const TI* proj, int nsplit, size_t split_stride,
+                                                 size_t row_stride, int col0, float* state,
+                                                 size_t state_stride, size_t tail_offset,
+                                                 const int32_t* seq_in, const int32_t* seq_out,
+                                                 const int32_t* seq_count, const int32_t* seq_row0,
+                                                 int n_seqs, int C, int J, size_t idx) {
   const size_t per_seq = static_cast<size_t>(J - 1) * C;
   if (idx >= static_cast<size_t>(n_seqs) * per_seq) return;
   const int seq = static_cast<int>(idx / per_seq);
@@ -297,15 +315,10 @@ extern "C" int ei_ssm_conv(const void* proj, int in_dtype, int nsplit, long long
   const size_t ss = static_cast<size_t>(split_stride), rs = static_cast<size_t>(row_stride);
   const size_t st = static_cast<size_t>(state_stride);
 #define EI_SSM_CONV(TI)                                                                          \
-  do {                                                                                           \
-    ssm_conv_kernel<TI><<<blocks, threads, 0, stream>>>(                                         \
-        static_cast<const TI*>(proj), nsplit, ss, rs, inner, w, bias, state, st, tail_offset,    \
-        row_pos, row_seq, seq_in, seq_start, conv, N, C, taps);                                  \
-    if (taps > 1)                                                                                \
-      ssm_tail_kernel<TI><<<tail_blocks, threads, 0, stream>>>(                                  \
-          static_cast<const TI*>(proj), nsplit, ss, rs, inner, state, st, tail_offset, seq_in,   \
-          seq_out, seq_count, seq_row0, n_seqs, C, taps);                                        \
-  } while (0)
+  ssm_conv_kernel<TI><<<blocks + (taps > 1 ? tail_blocks : 0), threads, 0, stream>>>(            \
+      static_cast<const TI*>(proj), nsplit, ss, rs, inner, w, bias, state, st, tail_offset,      \
+      row_pos, row_seq, seq_in, seq_start, conv, N, C, taps, state, seq_out, seq_count,          \
+      seq_row0, n_seqs, blocks)
   if (in_dtype == EI_F32) EI_SSM_CONV(float);
   else if (in_dtype == EI_BF16) EI_SSM_CONV(bf16_t);
   else EI_REQUIRE(false, "ssm_conv: unknown dtype");
