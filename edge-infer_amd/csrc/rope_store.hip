@@ -717,6 +717,115 @@ __global__ void head_store_kernel(
   }
 }
 
+
+template <typename TI>
+__device__ __forceinline__ void sliced8(const TI* p, int nsplit, size_t split_stride, float (&v)[8]) {
+  ei::VecN<TI, 8>::load(p, v);
+  for (int s = 1; s < nsplit; ++s) {
+    float more[8];
+    ei::VecN<TI, 8>::load(p + s * split_stride, more);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] += more[i];
+  }
+}
+
+// The same in 16-byte pieces, for head sizes, rotated halves and strides that are multiples of
+// 8: a lane takes 8 neighbouring elements, the G lanes of a head (G the power of two at or
+// above the widest head's eighth) add their squares by shuffles, and a wave takes 64 / G
+// (row, head) pairs.
+template <typename TI, typename TO>
+__global__ void head_store_vec_kernel(
+    const TI* __restrict__ proj, int nsplit, size_t split_stride, size_t row_stride,
+    const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w, float eps,
+    const double* __restrict__ freqs, int R, const int32_t* __restrict__ row_pos,
+    const int32_t* __restrict__ row_seq, const int32_t* __restrict__ page_table, int table_width,
+    TO* __restrict__ q_out, TO* __restrict__ k_pages, TO* __restrict__ v_pages,
+    float* __restrict__ v_first, int v_mode, const float* __restrict__ v_lambda,
+    int N, int nq, int nkv, int D, int DV, int write_cache, int G) {
+  const int heads = nq + 2 * nkv;
+  const size_t thread = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const size_t item = thread / G;
+  const int j = static_cast<int>(thread % G);                 // which eighth of the head
+  const bool in_range = item < static_cast<size_t>(N) * heads;
+  const int row = in_range ? static_cast<int>(item / heads) : 0;
+  const int head = in_range ? static_cast<int>(item % heads) : 0;
+  const int seq = in_range ? row_seq[row] : -1;
+  const bool is_q = head < nq, is_v = head >= nq + nkv;
+  // (every lane stays for the shuffles; `live` says whether it has anything to do)
+  const bool live = seq >= 0 && (is_q || write_cache || (is_v && v_mode == 1)) &&
+                    j * 8 < (is_v ? DV : D);
+  const int pos = seq >= 0 ? row_pos[row] : 0;
+  const TI* src_row = proj + static_cast<size_t>(row) * row_stride;
+  size_t page = 0;
+  if (live && write_cache)
+    page = static_cast<size_t>(page_table[static_cast<size_t>(seq) * table_width + pos / EI_PAGE]);
+  float x[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  if (is_v) {
+    if (!live) return;          // (value heads take no part in any shuffle: whole groups leave)
+    const int h = head - nq - nkv;
+    sliced8(src_row + static_cast<size_t>(nq + nkv) * D + static_cast<size_t>(h) * DV + j * 8, nsplit,
+            split_stride, x);
+    if (v_mode) {
+      float* first = v_first + static_cast<size_t>(row) * nkv * DV + static_cast<size_t>(h) * DV + j * 8;
+      if (v_mode == 1) {
+        ei::VecN<float, 8>::store(first, x);
+      } else {
+        const float lambda = *v_lambda;
+        float kept[8];
+        ei::VecN<float, 8>::load(first, kept);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[i] = (1.0f - lambda) * x[i] + lambda * kept[i];
+      }
+    }
+    if (write_cache)
+      ei::VecN<TO, 8>::store(
+          v_pages + ((page * nkv + h) * EI_PAGE + pos % EI_PAGE) * static_cast<size_t>(DV) + j * 8, x);
+    return;
+  }
+  const TI* src = src_row + static_cast<size_t>(head) * D;
+  const float* w = is_q ? q_norm_w : k_norm_w;
+  const int e0 = j * 8, rhalf = R / 2;
+  const bool turns = live && e0 < R;
+  const int partner0 = e0 < rhalf ? e0 + rhalf : e0 - rhalf;
+  float y[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  if (live) sliced8(src + e0, nsplit, split_stride, x);
+  if (turns) sliced8(src + partner0, nsplit, split_stride, y);
+  float inv = 1.0f;
+  if (w) {                      // (uniform: every lane of the wave takes the shuffles)
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) sum += x[i] * x[i];
+    for (int offset = G / 2; offset > 0; offset >>= 1) sum += __shfl_xor(sum, offset, EI_WAVE);
+    inv = 1.0f / sqrtf(sum / static_cast<float>(D) + eps);
+  }
+  if (!live) return;
+  if (w) {
+    float wx[8];
+    ei::VecN<float, 8>::load(w + e0, wx);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) x[i] = (x[i] * inv) * wx[i];
+    if (turns) {
+      ei::VecN<float, 8>::load(w + partner0, wx);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) y[i] = (y[i] * inv) * wx[i];
+    }
+  }
+  if (turns) {
+    const int f0 = e0 < rhalf ? e0 : e0 - rhalf;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const double whole = static_cast<double>(pos) * freqs[f0 + i] * 0.15915494309189535;
+      const float angle = static_cast<float>((whole - floor(whole)) * 6.283185307179586);
+      float sn, cs;
+      sincosf(angle, &sn, &cs);
+      x[i] = e0 < rhalf ? x[i] * cs - y[i] * sn : x[i] * cs + y[i] * sn;
+    }
+  }
+  TO* dst = is_q ? q_out + (static_cast<size_t>(row) * nq + head) * D
+                 : k_pages + ((page * nkv + (head - nq)) * EI_PAGE + pos % EI_PAGE) * static_cast<size_t>(D);
+  ei::VecN<TO, 8>::store(dst + e0, x);
+}
+
 }  // namespace
 
 extern "C" int ei_head_store(
@@ -743,6 +852,28 @@ extern "C" int ei_head_store(
   const size_t waves = static_cast<size_t>(N) * heads;
   const unsigned blocks = static_cast<unsigned>((waves * EI_WAVE + threads - 1) / threads);
   const size_t ss = static_cast<size_t>(split_stride), rs = static_cast<size_t>(row_stride);
+  // 16-byte pieces where every head, rotated half and stride is a multiple of 8
+  const auto aligned16 = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+  const bool vec = D % 8 == 0 && DV % 8 == 0 && R % 16 == 0 && rs % 8 == 0 && (nsplit == 1 || ss % 8 == 0) &&
+                   aligned16(proj) && aligned16(q_out) && aligned16(k_pages) && aligned16(v_pages) &&
+                   aligned16(v_first) && aligned16(q_norm_w) && aligned16(k_norm_w);
+  if (vec) {
+    int G = 1;
+    while (G * 8 < (D > DV ? D : DV)) G *= 2;
+    const size_t lanes = waves * G;
+    const unsigned vblocks = static_cast<unsigned>((lanes + threads - 1) / threads);
+#define EI_HSV(TI, TO)                                                                         \
+  head_store_vec_kernel<TI, TO><<<vblocks, threads, 0, stream>>>(                              \
+      static_cast<const TI*>(proj), nsplit, ss, rs, q_norm_w, k_norm_w, eps, freqs, R, row_pos, \
+      row_seq, page_table, table_width, static_cast<TO*>(q_out), static_cast<TO*>(k_pages),    \
+      static_cast<TO*>(v_pages), v_first, v_mode, v_lambda, N, nq, nkv, D, DV, write_cache, G)
+    if (in_dtype == EI_F32 && out_dtype == EI_F32) EI_HSV(float, float);
+    else if (in_dtype == EI_F32 && out_dtype == EI_BF16) EI_HSV(float, bf16_t);
+    else if (in_dtype == EI_BF16 && out_dtype == EI_BF16) EI_HSV(bf16_t, bf16_t);
+    else EI_REQUIRE(false, "head_store: unsupported dtype combination");
+#undef EI_HSV
+    EI_LAUNCH_CHECK();
+  }
 #define EI_HS(TI, TO)                                                                          \
   head_store_kernel<TI, TO><<<blocks, threads, 0, stream>>>(                                   \
       static_cast<const TI*>(proj), nsplit, ss, rs, q_norm_w, k_norm_w, eps, freqs, R, row_pos, \

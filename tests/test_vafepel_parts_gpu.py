@@ -182,15 +182,18 @@ def test_rescaled_frequencies_follow_the_three_cases():
 
 
 @pytest.mark.parametrize("heads, kv_heads, dim, vdim, rot_dims", [
-    (4, 2, 16, 24, 8), (3, 3, 10, 7, 10), (2, 1, 72, 8, 2), (5, 1, 12, 40, 0)])
+    (4, 2, 16, 24, 8), (3, 3, 10, 7, 10), (2, 1, 72, 8, 2), (5, 1, 12, 40, 0),
+    # sizes that take the kernel's form in 16-byte pieces (the rows then go on by 16 columns)
+    (4, 2, 64, 32, 16), (2, 2, 128, 128, 64), (3, 1, 24, 40, 0), (6, 3, 48, 8, 48)])
 @pytest.mark.parametrize("slices", [1, 2])
 def test_store_kernel(heads, kv_heads, dim, vdim, rot_dims, slices):
     """Queries out, keys and values in their pages: per-head norms, rotation of the first
     rot_dims elements at positions up to a million, values mixed with an earlier layer's, from
-    rows that go on after the values."""
+    rows that go on after the values (by 13 columns, or by 16 where all sizes are multiples
+    of 8)."""
     from edge_infer_amd.csrc import lib
     torch.manual_seed(heads * 100 + dim)
-    n_pages, tail = 10, 13
+    n_pages, tail = 10, (16 if dim % 8 == 0 and vdim % 8 == 0 else 13)
     qw, kw, vw = heads * dim, kv_heads * dim, kv_heads * vdim
     far = torch.tensor([0, 1, 63, 64, 65, 130, 1000000, 99999, 255, 300])     # the rows' positions
     n = far.numel()
