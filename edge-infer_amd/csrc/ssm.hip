@@ -124,9 +124,12 @@ constexpr int kScanTile = 16;     // tokens staged through LDS at a time
 constexpr int kScanThreads = 256;
 
 // A block a (sequence, head, block of columns of S).  A thread owns kScanRows rows of one
-// column; the L = Npad / kScanRows lanes of a column add their partial read-outs, a tile's
-// tokens side by side once the tile is walked, so that only S is a chain from token to token.
-template <typename TI>
+// column; the L = Npad / kScanRows lanes of a column add their partial read-outs with DPP adds,
+// and a token's operands are read from LDS while the token before it multiplies.
+// AHEAD: the next tile's rows are asked for from global memory before this tile is walked
+// (for launches of few blocks, where nothing else hides those reads; it costs registers, and
+// with them waves a SIMD where the chip is full).
+template <typename TI, bool AHEAD>
 __global__ void __launch_bounds__(kScanThreads)
 ssm_scan_kernel(const float* __restrict__ conv, const TI* __restrict__ proj, int nsplit,
                 size_t split_stride, size_t row_stride, int dt_col0,
@@ -175,60 +178,124 @@ ssm_scan_kernel(const float* __restrict__ conv, const TI* __restrict__ proj, int
   const float rate = expf(a_log[head]), bias = dt_bias[head], skip = d_skip[head];
   const int row0 = seq_row0[seq];
 
-  for (int t0 = 0; t0 < count; t0 += kScanTile) {
-    const int nt = min(kScanTile, count - t0);
-    __syncthreads();
-    for (int i = tid; i < nt * cols; i += kScanThreads) {
-      const int t = i / cols, cl = i % cols, c = blockIdx.z * cols + cl;
-      xs[i] = c < P ? conv[static_cast<size_t>(row0 + t0 + t) * C + head * P + c] : 0.f;
+  // Where the sizes allow 16-byte pieces and a thread's share of a tile is at most four of them
+  // an array, the next tile's rows are asked for from global memory before this tile is walked
+  // and go to LDS after it: the walk, not the reads, is then what a tile takes.
+  const int quads = npad / 4;                   // 16-byte pieces of a token's B (or C) in LDS
+  constexpr bool ahead = AHEAD;      // (the host has checked the sizes)
+  float4 pb[4], pc[4];
+  float px[4], pz = 0.f;
+  auto ask = [&](int t0n) {
+    const int ntn = min(kScanTile, count - t0n);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int i = tid + u * kScanThreads;
+      pb[u] = pc[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (i < ntn * quads) {
+        const int t = i / quads, n = (i % quads) * 4;
+        const float* src = conv + static_cast<size_t>(row0 + t0n + t) * C + inner + group * Nst;
+        if (n < Nst) {
+          pb[u] = *reinterpret_cast<const float4*>(src + n);
+          pc[u] = *reinterpret_cast<const float4*>(src + groups * Nst + n);
+        }
+      }
+      px[u] = 0.f;
+      if (i < ntn * cols) {
+        const int t = i / cols, c = blockIdx.z * cols + i % cols;
+        if (c < P) px[u] = conv[static_cast<size_t>(row0 + t0n + t) * C + head * P + c];
+      }
     }
-    for (int i = tid; i < nt * npad; i += kScanThreads) {
-      const int t = i / npad, n = i % npad;
-      const float* src = conv + static_cast<size_t>(row0 + t0 + t) * C + inner + group * Nst;
-      bs[i] = n < Nst ? src[n] : 0.f;
-      cs[i] = n < Nst ? src[groups * Nst + n] : 0.f;
+    if (tid < ntn)
+      pz = sliced(proj + static_cast<size_t>(row0 + t0n + tid) * row_stride + dt_col0 + head, nsplit,
+                  split_stride);
+  };
+  auto put = [&](int ntc) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int i = tid + u * kScanThreads;
+      if (i < ntc * quads) {
+        *reinterpret_cast<float4*>(bs + 4 * i) = pb[u];
+        *reinterpret_cast<float4*>(cs + 4 * i) = pc[u];
+      }
+      if (i < ntc * cols) xs[i] = px[u];
     }
-    if (tid < nt) {
-      const float z = sliced(proj + static_cast<size_t>(row0 + t0 + tid) * row_stride + dt_col0 + head,
-                             nsplit, split_stride) + bias;
+    if (tid < ntc) {
+      const float z = pz + bias;
       const float dt = z > 20.f ? z : log1pf(expf(z));
       dts[tid] = dt;
       decays[tid] = expf(-rate * dt);
     }
+  };
+  if constexpr (ahead) ask(0);
+
+  for (int t0 = 0; t0 < count; t0 += kScanTile) {
+    const int nt = min(kScanTile, count - t0);
     __syncthreads();
-    float sums[kScanTile];
-#pragma unroll
-    for (int t = 0; t < kScanTile; ++t) {
-      sums[t] = 0.f;
-      if (t >= nt) continue;
-      const float dt = dts[t], decay = decays[t];
-      const float x = xs[t * cols + col_local];
-      const float xdt = x * dt;
-      const float* b = bs + t * npad + n0;
-      const float* c = cs + t * npad + n0;
-      float acc = 0.f;
-#pragma unroll
-      for (int r = 0; r < kScanRows; r += 4) {
-        const float4 bv = *reinterpret_cast<const float4*>(b + r);
-        const float4 cv = *reinterpret_cast<const float4*>(c + r);
-        S[r] = decay * S[r] + bv.x * xdt;
-        S[r + 1] = decay * S[r + 1] + bv.y * xdt;
-        S[r + 2] = decay * S[r + 2] + bv.z * xdt;
-        S[r + 3] = decay * S[r + 3] + bv.w * xdt;
-        acc += S[r] * cv.x;
-        acc += S[r + 1] * cv.y;
-        acc += S[r + 2] * cv.z;
-        acc += S[r + 3] * cv.w;
+    if constexpr (ahead) {
+      put(nt);
+      if (t0 + kScanTile < count) ask(t0 + kScanTile);
+    } else {
+      for (int i = tid; i < nt * cols; i += kScanThreads) {
+        const int t = i / cols, cl = i % cols, c = blockIdx.z * cols + cl;
+        xs[i] = c < P ? conv[static_cast<size_t>(row0 + t0 + t) * C + head * P + c] : 0.f;
       }
-      sums[t] = acc;
+      for (int i = tid; i < nt * npad; i += kScanThreads) {
+        const int t = i / npad, n = i % npad;
+        const float* src = conv + static_cast<size_t>(row0 + t0 + t) * C + inner + group * Nst;
+        bs[i] = n < Nst ? src[n] : 0.f;
+        cs[i] = n < Nst ? src[groups * Nst + n] : 0.f;
+      }
+      if (tid < nt) {
+        const float z = sliced(proj + static_cast<size_t>(row0 + t0 + tid) * row_stride + dt_col0 + head,
+                               nsplit, split_stride) + bias;
+        const float dt = z > 20.f ? z : log1pf(expf(z));
+        dts[tid] = dt;
+        decays[tid] = expf(-rate * dt);
+      }
     }
+    __syncthreads();
+    // Two sets of a token's operands take turns: the LDS reads of the next token are asked
+    // for before this one multiplies, so a token waits for no read of its own.
+    float4 b0[4], c0[4], b1[4], c1[4];
+    float decay0, xdt0, x0, decay1, xdt1, x1;
+    auto fetch = [&](int t, float4 (&b4)[4], float4 (&c4)[4], float& decay, float& xdt, float& xv) {
+      const int tt = min(t, nt - 1);               // (a token beyond the tile: read, never used)
+      const float* bp = bs + tt * npad + n0;
+      const float* cp = cs + tt * npad + n0;
 #pragma unroll
-    for (int t = 0; t < kScanTile; ++t) {
-      if (t >= nt) continue;
-      const float total = group_sum(sums[t], L);
+      for (int i = 0; i < 4; ++i) {
+        b4[i] = *reinterpret_cast<const float4*>(bp + 4 * i);
+        c4[i] = *reinterpret_cast<const float4*>(cp + 4 * i);
+      }
+      decay = decays[tt];
+      xv = xs[tt * cols + col_local];
+      xdt = xv * dts[tt];
+    };
+    auto step = [&](int t, const float4 (&b4)[4], const float4 (&c4)[4], float decay, float xdt, float xv) {
+      float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;   // four sums: no single chain of additions
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        S[4 * i] = decay * S[4 * i] + b4[i].x * xdt;
+        S[4 * i + 1] = decay * S[4 * i + 1] + b4[i].y * xdt;
+        S[4 * i + 2] = decay * S[4 * i + 2] + b4[i].z * xdt;
+        S[4 * i + 3] = decay * S[4 * i + 3] + b4[i].w * xdt;
+        a0 += S[4 * i] * c4[i].x;
+        a1 += S[4 * i + 1] * c4[i].y;
+        a2 += S[4 * i + 2] * c4[i].z;
+        a3 += S[4 * i + 3] * c4[i].w;
+      }
+      const float total = group_sum((a0 + a1) + (a2 + a3), L);
       if (live && sub == 0)
-        y_raw[static_cast<size_t>(row0 + t0 + t) * inner + head * P + col] =
-            total + skip * xs[t * cols + col_local];
+        y_raw[static_cast<size_t>(row0 + t0 + t) * inner + head * P + col] = total + skip * xv;
+    };
+    static_assert(kScanRows == 16, "the walk takes a thread's rows as four 16-byte pieces");
+    fetch(0, b0, c0, decay0, xdt0, x0);
+#pragma unroll 1
+    for (int t = 0; t < nt; t += 2) {
+      fetch(t + 1, b1, c1, decay1, xdt1, x1);
+      step(t, b0, c0, decay0, xdt0, x0);
+      fetch(t + 2, b0, c0, decay0, xdt0, x0);
+      if (t + 1 < nt) step(t + 1, b1, c1, decay1, xdt1, x1);
     }
   }
   if (live) {
@@ -345,12 +412,22 @@ extern "C" int ei_ssm_scan(const float* conv, const void* proj, int in_dtype, in
   const dim3 grid(n_seqs, heads, (P + cols - 1) / cols);
   const size_t ss = static_cast<size_t>(split_stride), rs = static_cast<size_t>(row_stride);
   const int dt_col0 = inner + C;
+  // rows asked for a tile ahead: 16-byte pieces, at most four of them an array and thread, and a
+  // launch of so few blocks that a compute unit holds at most one (measured at 64, 512 and
+  // 4,096 blocks: 1,076 -> 790, 306 -> 334 and 1,760 -> 2,640 us)
+  const bool ahead = L >= 4 && L <= 16 && Nst % 4 == 0 && inner % 4 == 0 && (groups * Nst) % 4 == 0 &&
+                     static_cast<long long>(grid.x) * grid.y * grid.z <= 1LL * ei_compute_units();
 #define EI_SSM_SCAN(TI)                                                                           \
   do {                                                                                            \
+    if (ahead) EI_SSM_SCAN_AS(TI, true);                                                          \
+    else EI_SSM_SCAN_AS(TI, false);                                                               \
+  } while (0)
+#define EI_SSM_SCAN_AS(TI, AHEAD)                                                                 \
+  do {                                                                                            \
     if (lds > 48 * 1024)                                                                          \
-      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&ssm_scan_kernel<TI>),              \
+      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&ssm_scan_kernel<TI, AHEAD>),       \
                                 hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)); \
-    ssm_scan_kernel<TI><<<grid, kScanThreads, lds, stream>>>(                                     \
+    ssm_scan_kernel<TI, AHEAD><<<grid, kScanThreads, lds, stream>>>(                              \
         conv, static_cast<const TI*>(proj), nsplit, ss, rs, dt_col0, a_log, dt_bias, d_skip,      \
         state, static_cast<size_t>(state_stride), seq_in, seq_out, seq_count, seq_row0, y_raw,    \
         heads, groups, P, Nst, L);                                                                \
@@ -359,6 +436,7 @@ extern "C" int ei_ssm_scan(const float* conv, const void* proj, int in_dtype, in
   else if (in_dtype == EI_BF16) EI_SSM_SCAN(bf16_t);
   else EI_REQUIRE(false, "ssm_scan: unknown dtype");
 #undef EI_SSM_SCAN
+#undef EI_SSM_SCAN_AS
   EI_LAUNCH_CHECK();
 }
 
