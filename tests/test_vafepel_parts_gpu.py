@@ -527,7 +527,7 @@ def test_of_equal_logits_the_lower_index_is_chosen():
 
 @pytest.mark.parametrize("experts, top, inter, width, rows", [
     (6, 2, 40, 48, 21), (9, 3, 13, 50, 21), (4, 1, 96, 64, 21), (5, 2, 128, 64, 3),
-    (3, 2, 192, 128, 700), (12, 3, 64, 192, 77), (4, 2, 256, 512, 5), (6, 1, 512, 256, 40)])
+    (3, 2, 192, 128, 700), (12, 3, 64, 192, 77), (4, 2, 256, 512, 5), (6, 1, 512, 256, 40), (4, 2, 256, 512, 2), (5, 3, 768, 256, 1)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_the_experts_of_a_rows_choice(experts, top, inter, width, rows, dtype):
     """The experts' kernels on the router kernel's own choice, against the plain expert run on
