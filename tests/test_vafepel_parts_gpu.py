@@ -398,7 +398,9 @@ def plain_ssm(params, spec, x):
     dict(n_heads=4, head_dim=12, state=16, groups=2, conv_taps=4, norm_parts=2),
     dict(n_heads=3, head_dim=5, state=19, groups=1, conv_taps=1, norm_parts=1),
     dict(n_heads=6, head_dim=40, state=130, groups=3, conv_taps=7, norm_parts=4),
-    dict(n_heads=2, head_dim=300, state=8, groups=2, conv_taps=2, norm_parts=3)])
+    dict(n_heads=2, head_dim=300, state=8, groups=2, conv_taps=2, norm_parts=3),
+    dict(n_heads=2, head_dim=8, state=1024, groups=1, conv_taps=3, norm_parts=1),
+    dict(n_heads=4, head_dim=16, state=272, groups=2, conv_taps=4, norm_parts=2)])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_state_space_mixer_alone(shape, dtype):
     """Whole, in portions shorter than the convolution and down to two tokens, token by token."""
