@@ -111,7 +111,8 @@ class VafepelAttention:
         mask = _optional_object(source, "mask", where)
         if mask is not None:
             _known_keys(mask, ("size",), where + ".mask")
-            window = _int(mask, "size", where + ".mask")
+            if mask.get("size") is not None:          # (a mask without a size masks nothing)
+                window = _int(mask, "size", where + ".mask")
         rot = _optional_object(source, "rot", where)
         base, dims, scaling = None, 0, None
         if rot is not None:
@@ -282,7 +283,7 @@ class VafepelConfig:
                                   for index, layer in enumerate(layers)),
                      logit_scale=(1.0 if source.get("logit_scale") is None
                                   else _number(source, "logit_scale", "the top level")),
-                     logit_softcap=(None if source.get("logit_softcap") is None
+                     logit_softcap=(None if source.get("logit_softcap") in (None, 0, 0.0, False)
                                     else _number(source, "logit_softcap", "the top level")))
         widths = {layer.mixer.kv_heads * layer.mixer.vdim for layer in config.layers
                   if isinstance(layer.mixer, VafepelAttention) and layer.mixer.v_mix}

@@ -144,3 +144,6 @@ def test_what_may_be_absent():
         == ["off", "off", "off"]
     assert spec.layers[1].feed_forward is None and spec.layers[2].mixer.position.kind == "none"
     assert spec.layers[3].mixer.window is None
+    raw = edit(edit(CONFIGS["A"], ("layers", 0, "mixer", "mask", "size"), None), ("logit_softcap",), 0)
+    spec = config_class().from_dict(raw).model_spec()
+    assert spec.layers[0].mixer.window is None and spec.logit_softcap is None
