@@ -113,13 +113,16 @@ class SequencePages:
     that hold only positions no later query can see (position <= length - w)
     are given back; their table entries read -1.  `chunk` c: a query sees only keys of
     its own block of c positions (counted from the sequence's start), so pages that lie
-    wholly before the block of the next position are given back as well.
+    wholly before the block of the next position are given back as well.  `stride` s: the
+    group holds one entry for every complete block of s positions, so a sequence of n tokens
+    needs pages for n // s entries (such a group has no window and no chunk).
     """
 
-    def __init__(self, pool: PagePool, n_slots: int, window=None, chunk=None):
+    def __init__(self, pool: PagePool, n_slots: int, window=None, chunk=None, stride: int = 1):
         self.pool = pool
         self.window = window
         self.chunk = chunk
+        self.stride = max(1, int(stride))     # positions that share one entry of the group
         self._pages: Dict[int, List[int]] = {}
         self._version: Dict[int, int] = {}     # counts the changes of a slot's page list
         self._changes = 0
@@ -141,7 +144,7 @@ class SequencePages:
         return self._version[slot]
 
     def pages_needed(self, slot: int, new_length: int) -> int:
-        return max(0, pages_for(new_length) - len(self._pages[slot]))
+        return max(0, pages_for(new_length // self.stride) - len(self._pages[slot]))
 
     def grow(self, slot: int, new_length: int) -> None:
         need = self.pages_needed(slot, new_length)

@@ -38,26 +38,42 @@ class CacheLayout:
     def __init__(self, spec):
         self.kv_groups: List[Tuple[KVRequest, List[int]]] = []
         self.state_groups: List[Tuple[StateRequest, List[int]]] = []
-        self.entry_group: Dict[int, Tuple[str, int, int]] = {}  # cache id -> (kind, group, index)
+        # cache id (a schedule entry's, or (id, name) for a named thing of it) -> (kind, group, index)
+        self.entry_group: Dict[object, Tuple[str, int, int]] = {}
         for entry in spec.schedule:
-            if not entry.writes_cache:
-                continue
             layer = spec.layers[entry.layer]
             block_cls = lookup("block", layer.block)
             mixer_spec = block_cls.mixer_spec(layer)
-            request = lookup("mixer", mixer_spec.kind).cache_request(mixer_spec)
-            if request is None:
-                continue
-            groups = self.kv_groups if isinstance(request, KVRequest) else self.state_groups
-            kind = "kv" if isinstance(request, KVRequest) else "state"
-            for index, (held, entries) in enumerate(groups):
-                if held == request:
-                    self.entry_group[entry.cache] = (kind, index, len(entries))
-                    entries.append(entry.cache)
-                    break
-            else:
-                self.entry_group[entry.cache] = (kind, len(groups), 0)
-                groups.append((request, [entry.cache]))
+            mixer_cls = lookup("mixer", mixer_spec.kind)
+            if entry.writes_cache:
+                self._add(entry.cache, mixer_cls.cache_request(mixer_spec))
+            # what the run keeps for itself whichever cache entry its mixer reads: the state
+            # of its block arrangement, and what its mixer derives from another run's keys
+            own = getattr(block_cls, "own_cache_request", None)
+            if own is not None:
+                self._add(entry.own_id, own(layer))
+            own = getattr(mixer_cls, "own_cache_request", None)
+            if own is not None:
+                self._add(entry.own_id, own(mixer_spec))
+
+    def _add(self, cache_id, request) -> None:
+        if request is None:
+            return
+        if isinstance(request, dict):
+            for name, inner in request.items():
+                self._add(cache_id if name == "" else (cache_id, name), inner)
+            return
+        if cache_id in self.entry_group:
+            raise ValueError(f"cache entry {cache_id!r} is asked for twice")
+        groups = self.kv_groups if isinstance(request, KVRequest) else self.state_groups
+        kind = "kv" if isinstance(request, KVRequest) else "state"
+        for index, (held, entries) in enumerate(groups):
+            if held == request:
+                self.entry_group[cache_id] = (kind, index, len(entries))
+                entries.append(cache_id)
+                return
+        self.entry_group[cache_id] = (kind, len(groups), 0)
+        groups.append((request, [cache_id]))
 
 
 class SessionCache:
@@ -77,11 +93,14 @@ class SessionCache:
         self.kv_k: List[torch.Tensor] = []
         self.kv_v: List[torch.Tensor] = []
         for request, entries in layout.kv_groups:
-            pool = PagePool(self.n_pages)
+            # a group that holds one entry a block of `stride` positions needs that much less:
+            # the tokens' share, and a partly filled last page for every sequence
+            pool = PagePool(self.n_pages if request.stride <= 1 else
+                            min(self.n_pages, self.n_pages // request.stride + self.n_slots + 1))
             self.kv_pools.append(pool)
             self.kv_pages.append(SequencePages(pool, self.n_slots, window=request.window,
-                                               chunk=request.chunk))
-            shape = (len(entries), self.n_pages, request.n_kv_heads, PAGE_TOKENS)
+                                               chunk=request.chunk, stride=request.stride))
+            shape = (len(entries), pool.n_pages, request.n_kv_heads, PAGE_TOKENS)
             value_dim = request.head_dim if request.value_dim is None else request.value_dim
             self.kv_k.append(torch.empty(shape + (request.head_dim,), dtype=dtype, device=device))
             self.kv_v.append(torch.empty(shape + (value_dim,), dtype=dtype, device=device))

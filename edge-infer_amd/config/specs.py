@@ -15,6 +15,8 @@ from typing import Optional, Tuple
 
 @dataclass(frozen=True)
 class NormSpec:
+    """kind "rmsnorm": x / sqrt(mean(x^2) + eps) * w; kind "layernorm":
+    (x - mean) / sqrt(mean((x - mean)^2) + eps) * w + b, with a weight and a bias."""
     kind: str = "rmsnorm"
     eps: float = 1e-6
 
@@ -89,8 +91,23 @@ class AttentionSpec:
     # checkpoint may hold the (unused) number; None: no such thing
     value_mix: Optional[str] = None
     # the concatenated heads are multiplied, element by element, by sigmoid(W_g x), x the
-    # mixer's input, before the output projection
-    output_gate: bool = False
+    # mixer's input, before the output projection; "head": W_g has one row a head, and every
+    # element of a head's output is multiplied by that head's sigmoid
+    output_gate: object = False
+    # P: besides the tokens of its window a query at position i sees one key and value for
+    # every block b of P positions that lies wholly before the window (b P + P - 1 <= i -
+    # window): the means of the block's cached keys and of its values; tokens and blocks share
+    # one softmax.  Needs a window.
+    pool: Optional[int] = None
+    # (coef, every): the query at position p is multiplied by
+    # 1 + coef ln(floor((p + 1) / every) + 1)
+    query_temperature: Optional[Tuple[float, int]] = None
+    # the part has no key and value projections: every run of it reads keys and values that
+    # another run has cached (its schedule entries never write the cache)
+    shared_kv: bool = False
+    # positions behind the newest one that the cache keeps for other runs that read it with a
+    # wider mask than this layer's own: None: what the own window and pool need; 0: all
+    cache_span: Optional[int] = None
 
     @property
     def q_width(self) -> int:
@@ -132,11 +149,24 @@ class GatedMLPSpec:
 class RoutedMLPSpec:
     """Mixture of experts: a router chooses `top` of `n_experts` gated feed-forwards
     down(silu(gate x) * up x) for every token, by the largest float32 logits W_router x, and
-    adds their outputs weighted by the softmax over the chosen logits alone."""
+    adds their outputs weighted by the softmax over the chosen logits alone.
+
+    `scoring` "softmax_all": the scores are the softmax over all router outputs, the choice is
+    by the largest score (plus a learned per-output `correction` where the spec says so), and
+    the weights are the chosen scores themselves, not renormalised.  `identity`: the router
+    has that many outputs beyond `n_experts`; one of them chosen adds the input row itself,
+    times its weight (such experts have no matrices)."""
     kind: str = "routed_mlp"
     n_experts: int = 0
     top: int = 0
     intermediate_size: int = 0    # of one expert
+    scoring: str = "softmax_chosen"
+    correction: bool = False
+    identity: int = 0
+
+    @property
+    def router_outputs(self) -> int:
+        return self.n_experts + self.identity
 
 
 @dataclass(frozen=True)
@@ -156,6 +186,39 @@ class StateSpaceSpec:
     @property
     def inner(self) -> int:
         return self.n_heads * self.head_dim
+
+
+@dataclass(frozen=True)
+class LinearAttentionSpec:
+    """Linear attention with a fixed decay per head: q = silu(W_q x), k = silu(W_k x) (heads x
+    key_dim), v = silu(W_v x) (heads x value_dim); per head S_t = decay_h S_(t-1) + k_t v_t^T
+    and o_t = S_t^T q_t; the concatenated heads pass an RMS norm with a weight, are multiplied
+    by sigmoid(W_g x), and projected.  See `parts.linear_attention`."""
+    kind: str = "linear_attention"
+    n_heads: int = 0
+    key_dim: int = 0
+    value_dim: int = 0
+    decay: Tuple[float, ...] = ()     # one per head
+    norm_eps: float = 1e-6
+
+    @property
+    def qk_width(self) -> int:
+        return self.n_heads * self.key_dim
+
+    @property
+    def v_width(self) -> int:
+        return self.n_heads * self.value_dim
+
+
+@dataclass(frozen=True)
+class ParallelSpec:
+    """Several mixers side by side that read the same rows: the result is the mean of their
+    outputs, each first RMS-normed over the model's width with a weight of its own.  See
+    `parts.parallel`."""
+    kind: str = "parallel"
+    branches: Tuple[object, ...] = ()     # mixer specs
+    names: Tuple[str, ...] = ()           # parameter prefix of every branch
+    norm_eps: float = 1e-6
 
 
 @dataclass(frozen=True)
@@ -251,6 +314,16 @@ class LayerSpec:
     feed_forward: object  # a spec with a .kind (GatedMLPSpec, ...), or None: no feed-forward
     # what a sublayer adds to the stream is multiplied by this (arrangements that know it)
     residual_scale: float = 1.0
+    # what a sublayer adds is multiplied, element by element, by a learned vector of the
+    # model's width, one for the mixer and one for the feed-forward (arrangements that know it)
+    layer_scale: bool = False
+    # taps T > 0: what a sublayer reads, h, is replaced by h + conv(h), a causal convolution
+    # over time on every channel with a learned filter [width, T] per sublayer and no bias:
+    # conv(h)_t = sum_j w[:, j] h_(t - T + 1 + j), zeros before the sequence's start; the last
+    # T - 1 inputs of both sublayers are state of the sequence (arrangements that know it)
+    input_conv: int = 0
+    # the model's width, for arrangements that ask for state of that width (None: not needed)
+    width: Optional[int] = None
 
 
 @dataclass(frozen=True)
@@ -267,10 +340,17 @@ class LoopSpec:
 @dataclass(frozen=True)
 class ScheduleEntry:
     """One run of a layer.  `cache` is the id of the cache entry the mixer uses;
-    `writes_cache` False means it only reads an entry that another run wrote."""
+    `writes_cache` False means it only reads an entry that another run wrote.  `own` is the id
+    under which the run keeps what is its own whatever `cache` says (the state of its block,
+    what its mixer derives from keys that another run wrote); None: the same as `cache`."""
     layer: int
     cache: int
     writes_cache: bool = True
+    own: Optional[int] = None
+
+    @property
+    def own_id(self) -> int:
+        return self.cache if self.own is None else self.own
 
 
 @dataclass(frozen=True)
@@ -302,6 +382,17 @@ class ModelSpec:
                 if entry.cache in writers:
                     raise ValueError(f"cache entry {entry.cache} has two writers")
                 writers[entry.cache] = entry.layer
+        owners = {}
+        for run, entry in enumerate(self.schedule):
+            if entry.own is None:
+                continue
+            # what a run keeps under `own` must not be another run's
+            if entry.own in owners or (entry.own in writers and entry.own != entry.cache) \
+                    or any(other.cache == entry.own or other.own == entry.own
+                           for index, other in enumerate(self.schedule) if index != run):
+                raise ValueError(f"the id {entry.own} under which run {run} keeps its own "
+                                 "state is also another run's")
+            owners[entry.own] = run
         if self.loop is not None:
             loop = self.loop
             if not (0 <= loop.start < loop.stop <= len(self.layers)) or loop.times < 1:

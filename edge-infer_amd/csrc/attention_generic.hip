@@ -15,7 +15,10 @@
 // how scores mixed over heads are taken: a mix of scores is the score of mixed queries;
 // values still come from the row's own kv head), `values_in_keys` (the values are the first DV
 // elements of the key rows: a latent that serves as key and value is cached once), `gate` (per
-// row and head: the output is multiplied by sigmoid(gate)).
+// row and head: the output is multiplied by sigmoid(gate)), `pool` (with a window w: besides the
+// tokens of its window a query at p sees entry b of a second paged cache, which holds one key and
+// value for every block of `pool` positions, if b pool + pool - 1 <= p - w; tokens and blocks
+// share one softmax).
 // operators/src/cuda/execution.cu:137-179, runtime/src/qwen.cpp:374-402,
 // split merge: operators/src/cuda/kernels/gather_fa_variable.cu:14-118.
 #include "common.h"
@@ -39,7 +42,8 @@ attn_generic_kernel(const T* __restrict__ q, const T* __restrict__ k_pages,
                     int head_blocks, int BC, int window, int chunk,
                     const float* __restrict__ slopes, const float* __restrict__ sinks,
                     float scale, int n_splits, int KH, int values_in_keys,
-                    const float* __restrict__ gate) {
+                    const float* __restrict__ gate, int pool, const T* __restrict__ pool_k,
+                    const T* __restrict__ pool_v, const int32_t* __restrict__ pool_table) {
   extern __shared__ float lds[];
   const int DQ = KH * D;                  // width of a query row and of a key as it is met
   float* Qs = lds;                        // [kRows][DQ]
@@ -82,6 +86,85 @@ attn_generic_kernel(const T* __restrict__ q, const T* __restrict__ k_pages,
   const int nd = (DV + 15) / 16;
   const int nj = BC / 16;
 
+  // pooled blocks that this row sees: those wholly before its window
+  const int blocks_r = (pool > 0 && window > 0 && row_valid && pos_r - window + 1 > 0)
+                           ? (pos_r - window + 1) / pool : 0;
+  // One chunk of BC keys (chunk `ch` of a page whose first key is key0; keys beyond last_key
+  // hold stale bytes) against the block's rows: scores, running maximum and sum, values.
+  auto walk = [&](const T* kp, const T* vp, int DVS, int phys, int ch, int key0, int last_key,
+                  bool pooled) {
+      __syncthreads();
+      for (int idx = t; idx < BC * DQ; idx += kThreads) {
+        const int c = idx / DQ, d = idx % DQ;
+        const bool live = key0 + c <= last_key;  // later slots hold stale bytes
+        // with key_heads > 1 the piece d / D of the key lies in that kv head's page part
+        const T* src = KH > 1 ? k_pages + (static_cast<size_t>(phys) * nkv + d / D) * EI_PAGE * D
+                              : kp;
+        const size_t off = static_cast<size_t>(ch * BC + c) * D + (KH > 1 ? d % D : d);
+        Ks[c * (DQ + 1) + d] = live ? ei::to_f32<T>(src[off]) : 0.f;
+      }
+      for (int idx = t; idx < BC * DV; idx += kThreads) {
+        const int c = idx / DV, d = idx % DV;
+        const bool live = key0 + c <= last_key;
+        const size_t off = static_cast<size_t>(ch * BC + c) * DVS + d;
+        Vs[c * DV + d] = live ? ei::to_f32<T>(vp[off]) : 0.f;
+      }
+      __syncthreads();
+      float s[4];
+      float row_max = kLowest;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        s[j] = -INFINITY;
+        if (j < nj) {
+          const int c = cc + 16 * j;
+          const int key = key0 + c;
+          const bool visible =
+              pooled ? (row_valid && key < blocks_r)
+                     : (row_valid && key <= pos_r && (window <= 0 || key > pos_r - window) &&
+                        (chunk <= 0 || key / chunk == chunk_r));
+          if (visible) {
+            float dot = 0.f;
+            const float* qr = Qs + r * DQ;
+            const float* kr = Ks + c * (DQ + 1);
+            for (int d = 0; d < DQ; ++d) dot += qr[d] * kr[d];
+            if (!pooled) dot -= slope * static_cast<float>(pos_r - key);
+            s[j] = dot;
+            row_max = fmaxf(row_max, dot);
+          }
+        }
+      }
+#pragma unroll
+      for (int offset = 8; offset > 0; offset >>= 1)
+        row_max = fmaxf(row_max, __shfl_xor(row_max, offset, 16));
+      const float m_new = fmaxf(m_r, row_max);
+      const float alpha = expf(m_r - m_new);
+      float row_sum = 0.f;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (j < nj) {
+          const float p_val = expf(s[j] - m_new);  // -inf -> 0
+          Ps[r * (BC + 1) + cc + 16 * j] = p_val;
+          row_sum += p_val;
+        }
+      }
+#pragma unroll
+      for (int offset = 8; offset > 0; offset >>= 1) row_sum += __shfl_xor(row_sum, offset, 16);
+      l_r = l_r * alpha + row_sum;
+      m_r = m_new;
+      __syncthreads();
+      const float* pr = Ps + r * (BC + 1);
+#pragma unroll
+      for (int k = 0; k < kAcc; ++k) {
+        if (k < nd) {
+          const int d = cc + 16 * k;
+          float a = acc[k] * alpha;
+          if (d < DV)
+            for (int c = 0; c < BC; ++c) a += pr[c] * Vs[c * DV + d];
+          acc[k] = a;
+        }
+      }
+  };
+
   if (seq >= 0 && npos > 0) {
     const int hi_key = row_pos[row0 + npos - 1];
     int lo_key = window > 0 ? max(0, row_pos[row0] - window + 1) : 0;
@@ -104,73 +187,24 @@ attn_generic_kernel(const T* __restrict__ q, const T* __restrict__ k_pages,
         const int key0 = p * EI_PAGE + ch * BC;
         if (key0 > hi_key) break;
         if (key0 + BC <= lo_key) continue;   // wholly before what any row of the item sees
-        __syncthreads();
-        for (int idx = t; idx < BC * DQ; idx += kThreads) {
-          const int c = idx / DQ, d = idx % DQ;
-          const bool live = key0 + c <= hi_key;  // later slots hold stale bytes
-          // with key_heads > 1 the piece d / D of the key lies in that kv head's page part
-          const T* src = KH > 1 ? k_pages + (static_cast<size_t>(phys) * nkv + d / D) * EI_PAGE * D
-                                : kp;
-          const size_t off = static_cast<size_t>(ch * BC + c) * D + (KH > 1 ? d % D : d);
-          Ks[c * (DQ + 1) + d] = live ? ei::to_f32<T>(src[off]) : 0.f;
-        }
-        for (int idx = t; idx < BC * DV; idx += kThreads) {
-          const int c = idx / DV, d = idx % DV;
-          const bool live = key0 + c <= hi_key;
-          const size_t off = static_cast<size_t>(ch * BC + c) * DVS + d;
-          Vs[c * DV + d] = live ? ei::to_f32<T>(vp[off]) : 0.f;
-        }
-        __syncthreads();
-        float s[4];
-        float row_max = kLowest;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          s[j] = -INFINITY;
-          if (j < nj) {
-            const int c = cc + 16 * j;
-            const int key = key0 + c;
-            const bool visible = row_valid && key <= pos_r && (window <= 0 || key > pos_r - window) &&
-                                 (chunk <= 0 || key / chunk == chunk_r);
-            if (visible) {
-              float dot = 0.f;
-              const float* qr = Qs + r * DQ;
-              const float* kr = Ks + c * (DQ + 1);
-              for (int d = 0; d < DQ; ++d) dot += qr[d] * kr[d];
-              dot -= slope * static_cast<float>(pos_r - key);
-              s[j] = dot;
-              row_max = fmaxf(row_max, dot);
-            }
-          }
-        }
-#pragma unroll
-        for (int offset = 8; offset > 0; offset >>= 1)
-          row_max = fmaxf(row_max, __shfl_xor(row_max, offset, 16));
-        const float m_new = fmaxf(m_r, row_max);
-        const float alpha = expf(m_r - m_new);
-        float row_sum = 0.f;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          if (j < nj) {
-            const float p_val = expf(s[j] - m_new);  // -inf -> 0
-            Ps[r * (BC + 1) + cc + 16 * j] = p_val;
-            row_sum += p_val;
-          }
-        }
-#pragma unroll
-        for (int offset = 8; offset > 0; offset >>= 1) row_sum += __shfl_xor(row_sum, offset, 16);
-        l_r = l_r * alpha + row_sum;
-        m_r = m_new;
-        __syncthreads();
-        const float* pr = Ps + r * (BC + 1);
-#pragma unroll
-        for (int k = 0; k < kAcc; ++k) {
-          if (k < nd) {
-            const int d = cc + 16 * k;
-            float a = acc[k] * alpha;
-            if (d < DV)
-              for (int c = 0; c < BC; ++c) a += pr[c] * Vs[c * DV + d];
-            acc[k] = a;
-          }
+        walk(kp, vp, DVS, phys, ch, key0, hi_key, false);
+      }
+    }
+    if (pool > 0 && window > 0) {
+      // the pooled blocks that the item's last row sees (its other rows see fewer): entries
+      // 0 .. seen - 1 of the pooled cache, whose pages the slices take in turn
+      const int before = hi_key - window + 1;
+      const int seen = before > 0 ? before / pool : 0;
+      const int pool_pages = (seen + EI_PAGE - 1) / EI_PAGE;
+      for (int p = split; p < pool_pages; p += n_splits) {
+        const int phys = pool_table[static_cast<size_t>(seq) * table_width + p];
+        if (phys < 0) continue;
+        const T* kp = pool_k + (static_cast<size_t>(phys) * nkv + g) * EI_PAGE * D;
+        const T* vp = pool_v + (static_cast<size_t>(phys) * nkv + g) * EI_PAGE * DV;
+        for (int ch = 0; ch < chunks_per_page; ++ch) {
+          const int key0 = p * EI_PAGE + ch * BC;
+          if (key0 >= seen) break;
+          walk(kp, vp, DV, phys, ch, key0, seen - 1, true);
         }
       }
     }
@@ -257,7 +291,8 @@ extern "C" int ei_attention(const void* q, const void* k_pages, const void* v_pa
                             void* out, float* part_o, float* part_ml, int N, int nq, int nkv,
                             int D, int DV, int window, int chunk, const float* slopes,
                             const float* sinks, float scale, int n_splits, int key_heads,
-                            int values_in_keys, const float* gate, hipStream_t stream) {
+                            int values_in_keys, const float* gate, int pool, const void* pool_k,
+                            const void* pool_v, const int32_t* pool_table, hipStream_t stream) {
   EI_REQUIRE(n_items > 0 && N > 0 && nq > 0 && nkv > 0, "attention: sizes must be positive");
   EI_REQUIRE(nq % nkv == 0, "attention: query heads must be a multiple of kv heads");
   EI_REQUIRE(key_heads == 1 || key_heads == nkv,
@@ -274,6 +309,9 @@ extern "C" int ei_attention(const void* q, const void* k_pages, const void* v_pa
   EI_REQUIRE(n_splits >= 1 && n_splits <= 64, "attention: splits must be between 1 and 64");
   EI_REQUIRE(n_splits == 1 || (part_o && part_ml), "attention: split scratch missing");
   EI_REQUIRE(window >= 0, "attention: negative window");
+  EI_REQUIRE(pool >= 0 && (pool == 0 || (window > 0 && pool_k && pool_v && pool_table &&
+                                         key_heads == 1 && !values_in_keys)),
+             "attention: pooled blocks need a window, their cache and keys of one kv head");
   const int G = nq / nkv;
   const int Gb = G < kRows ? G : kRows;
   const int head_blocks = (G + Gb - 1) / Gb;
@@ -303,13 +341,15 @@ extern "C" int ei_attention(const void* q, const void* k_pages, const void* v_pa
         static_cast<const float*>(q), static_cast<const float*>(k_pages),
         static_cast<const float*>(v_pages), item_seq, item_row0, item_npos, row_pos, page_table,
         table_width, static_cast<float*>(out), part_o, part_ml, nq, nkv, D, DV, Gb, head_blocks,
-        BC, window, chunk, slopes, sinks, scale, n_splits, key_heads, values_in_keys, gate);
+        BC, window, chunk, slopes, sinks, scale, n_splits, key_heads, values_in_keys, gate, pool,
+        static_cast<const float*>(pool_k), static_cast<const float*>(pool_v), pool_table);
   } else if (dtype == EI_BF16) {
     attn_generic_kernel<bf16_t><<<grid, kThreads, lds, stream>>>(
         static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pages),
         static_cast<const bf16_t*>(v_pages), item_seq, item_row0, item_npos, row_pos, page_table,
         table_width, static_cast<bf16_t*>(out), part_o, part_ml, nq, nkv, D, DV, Gb, head_blocks,
-        BC, window, chunk, slopes, sinks, scale, n_splits, key_heads, values_in_keys, gate);
+        BC, window, chunk, slopes, sinks, scale, n_splits, key_heads, values_in_keys, gate, pool,
+        static_cast<const bf16_t*>(pool_k), static_cast<const bf16_t*>(pool_v), pool_table);
   } else {
     EI_REQUIRE(false, "attention: unknown dtype");
   }
@@ -329,5 +369,81 @@ extern "C" int ei_attention(const void* q, const void* k_pages, const void* v_pa
       attn_merge_kernel<bf16_t><<<blocks, threads, 0, stream>>>(
           part_o, part_ml, row_seq, static_cast<bf16_t*>(out), nq, DV, n_splits, total, gate);
   }
+  EI_LAUNCH_CHECK();
+}
+
+// ---------------------------------------------------------------------------------------
+// The pooled cache: entry b holds the means of the cached keys and of the cached values of the
+// positions b P .. b P + P - 1 of a sequence, for every kv head.  A wave a (row, kv head): the
+// row at position p with (p + 1) % P == 0 completes block p / P, whose keys all lie in the
+// token cache by then (this step's store has run), and writes the block's entry; every other
+// row has nothing to do.  Sums are float32, in the order of the positions.
+namespace {
+
+template <typename T>
+__global__ void pool_store_kernel(const T* __restrict__ k_pages, const T* __restrict__ v_pages,
+                                  const int32_t* __restrict__ row_pos,
+                                  const int32_t* __restrict__ row_seq,
+                                  const int32_t* __restrict__ page_table,
+                                  const int32_t* __restrict__ pool_table, int table_width,
+                                  T* __restrict__ pool_k, T* __restrict__ pool_v, int N, int nkv,
+                                  int D, int DV, int P) {
+  const int wave = (blockIdx.x * blockDim.x + threadIdx.x) / EI_WAVE;
+  const int lane = threadIdx.x % EI_WAVE;
+  if (wave >= N * nkv) return;
+  const int row = wave / nkv, g = wave % nkv;
+  const int seq = row_seq[row];
+  if (seq < 0) return;
+  const int pos = row_pos[row];
+  if ((pos + 1) % P != 0) return;
+  const int block = pos / P;
+  const int32_t* pages = page_table + static_cast<size_t>(seq) * table_width;
+  const int dst_page = pool_table[static_cast<size_t>(seq) * table_width + block / EI_PAGE];
+  if (dst_page < 0) return;
+  const size_t dst = (static_cast<size_t>(dst_page) * nkv + g) * EI_PAGE + block % EI_PAGE;
+  const float share = 1.0f / static_cast<float>(P);
+  for (int e = lane; e < D + DV; e += EI_WAVE) {
+    const bool key = e < D;
+    const int width = key ? D : DV, at = key ? e : e - D;
+    const T* source = key ? k_pages : v_pages;
+    float sum = 0.f;
+    for (int j = 0; j < P; ++j) {
+      const int p = block * P + j;
+      const int phys = pages[p / EI_PAGE];
+      if (phys >= 0)
+        sum += ei::to_f32<T>(source[((static_cast<size_t>(phys) * nkv + g) * EI_PAGE + p % EI_PAGE) *
+                                    width + at]);
+    }
+    (key ? pool_k : pool_v)[dst * width + at] = ei::from_f32<T>(sum * share);
+  }
+}
+
+}  // namespace
+
+// k_pages [pages, nkv, 64, D], v_pages [pages, nkv, 64, DV] hold the tokens; pool_k, pool_v the
+// same shapes for the pooled entries, found through pool_table as tokens are through page_table.
+extern "C" int ei_pool_store(const void* k_pages, const void* v_pages, int dtype,
+                             const int32_t* row_pos, const int32_t* row_seq,
+                             const int32_t* page_table, const int32_t* pool_table, int table_width,
+                             void* pool_k, void* pool_v, int N, int nkv, int D, int DV, int P,
+                             hipStream_t stream) {
+  EI_REQUIRE(k_pages && v_pages && row_pos && row_seq && page_table && pool_table && pool_k && pool_v,
+             "pool_store: null pointer");
+  EI_REQUIRE(N > 0 && nkv > 0 && D > 0 && DV > 0 && P >= 1 && table_width > 0,
+             "pool_store: sizes must be positive");
+  const size_t waves = static_cast<size_t>(N) * nkv;
+  const unsigned blocks = static_cast<unsigned>((waves * EI_WAVE + 255) / 256);
+  if (dtype == EI_F32)
+    pool_store_kernel<float><<<blocks, 256, 0, stream>>>(
+        static_cast<const float*>(k_pages), static_cast<const float*>(v_pages), row_pos, row_seq,
+        page_table, pool_table, table_width, static_cast<float*>(pool_k),
+        static_cast<float*>(pool_v), N, nkv, D, DV, P);
+  else if (dtype == EI_BF16)
+    pool_store_kernel<bf16_t><<<blocks, 256, 0, stream>>>(
+        static_cast<const bf16_t*>(k_pages), static_cast<const bf16_t*>(v_pages), row_pos, row_seq,
+        page_table, pool_table, table_width, static_cast<bf16_t*>(pool_k),
+        static_cast<bf16_t*>(pool_v), N, nkv, D, DV, P);
+  else
+    EI_REQUIRE(false, "pool_store: unknown dtype");
   EI_LAUNCH_CHECK();
 }

@@ -21,7 +21,7 @@ from pathlib import Path
 SOURCE_DIR = Path(__file__).resolve().parent
 LIBRARIES = ("rowwise", "rope_store", "attention_generic", "attention_mfma", "gemm_f32",
              "gemm_bf16", "sampling", "peaks", "delta_rule", "head_ops", "mlstm", "attention_wide",
-             "ssm", "moe")
+             "ssm", "moe", "norms", "input_conv", "linear_attention")
 ARCH = "gfx950"
 # packed-fp32 instructions are switched off for every device compilation
 FLAGS = ("-O3", "-std=c++17", "-fPIC", "-shared", f"--offload-arch={ARCH}",

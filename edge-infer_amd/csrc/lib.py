@@ -55,7 +55,8 @@ _SIGNATURES = {
         "ei_head_store": [c_void_p, c_int, c_int, c_longlong, c_longlong, c_void_p, c_void_p,
                           c_float, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                           c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int,
-                          c_int, c_int, c_int, c_int, c_void_p],
+                          c_int, c_int, c_int, c_int, c_float, c_int, c_void_p, c_longlong,
+                          c_void_p],
         "ei_projection_norm_store": [c_void_p, c_int, c_int, c_longlong, c_void_p, c_void_p, c_void_p,
                                      c_float, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                      c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
@@ -73,11 +74,30 @@ _SIGNATURES = {
         "ei_ssm_out": [c_void_p, c_void_p, c_int, c_int, c_longlong, c_longlong, c_void_p,
                        c_float, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     },
+    "norms": {
+        "ei_stream_norm": [c_void_p, c_void_p, c_int, c_int, c_longlong, c_void_p, c_void_p,
+                           c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_int, c_void_p, c_int,
+                           c_int, c_int, c_int, c_void_p],
+        "ei_norm_mean": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_float,
+                         c_void_p, c_int, c_int, c_void_p],
+    },
+    "input_conv": {
+        "ei_input_conv": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p,
+                          c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                          c_int, c_int, c_int, c_void_p],
+    },
+    "linear_attention": {
+        "ei_la_scan": [c_void_p, c_int, c_int, c_longlong, c_longlong, c_void_p, c_void_p,
+                       c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                       c_int, c_void_p],
+        "ei_la_out": [c_void_p, c_void_p, c_int, c_int, c_longlong, c_longlong, c_longlong,
+                      c_void_p, c_float, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+    },
     "moe": {
         "ei_moe_route": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
-                         c_int, c_int, c_void_p],
+                         c_int, c_int, c_int, c_void_p, c_void_p],
         "ei_moe_experts": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
-                           c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+                           c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
         "ei_moe_grouped_supported": [c_int, c_int, c_int, c_int],
         "ei_moe_experts_grouped": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                    c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
@@ -103,7 +123,9 @@ _SIGNATURES = {
         "ei_attention": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
                          c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
                          c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float,
-                         c_int, c_int, c_int, c_void_p, c_void_p],
+                         c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p],
+        "ei_pool_store": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                          c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
     },
     "attention_wide": {
         "ei_attn_wide_supported": [c_int, c_int, c_int],
@@ -570,7 +592,8 @@ def attention_positions_per_item(group: int) -> int:
 def attention(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items, row_pos, row_seq,
               page_table, out, n_heads, n_kv_heads, head_dim, window=None, scale=None,
               n_splits=1, part_o=None, part_ml=None, value_dim=None, chunk=None, slopes=None,
-              sinks=None, key_heads=1, values_in_keys=False, gate=None) -> None:
+              sinks=None, key_heads=1, values_in_keys=False, gate=None, pool=None,
+              pool_k=None, pool_v=None, pool_table=None) -> None:
     """Generic causal attention over the paged cache (see attention_generic.hip).
     value_dim: head size of the values and of `out` (None: head_dim); chunk: a query sees only
     the keys of its own block of that many positions; slopes, sinks: float32 [n_heads], the
@@ -579,7 +602,9 @@ def attention(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items, row_
     keys of all kv heads of a position laid end to end (scores mixed over heads: see
     `mix_heads`).  values_in_keys: the values are the first value_dim elements of the key
     rows and `v_pages` is not read.  gate: float32 [rows, heads]; the output of a row and
-    head is multiplied by sigmoid(gate)."""
+    head is multiplied by sigmoid(gate).  pool: P (needs a window): a query also sees the
+    entries of the pooled cache (`pool_k`, `pool_v`: pages shaped like the tokens' pages, found
+    through `pool_table`) whose blocks of P positions lie wholly before its window."""
     lib = library("attention_generic")
     n = q.shape[0]
     value_dim = head_dim if value_dim is None else int(value_dim)
@@ -614,6 +639,13 @@ def attention(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items, row_
         if part_o is None or part_ml is None or part_o.numel() < need_o \
                 or part_ml.numel() < n * n_heads * n_splits * 2:
             raise KernelError("attention: split scratch missing or too small")
+    if pool:
+        if not window or pool_k is None or pool_v is None or pool_table is None:
+            raise KernelError("attention: pooled blocks need a window and their cache")
+        if tuple(pool_k.shape[1:]) != expect or tuple(pool_v.shape[1:]) != expect_v[1:] \
+                or pool_k.dtype != q.dtype or pool_v.dtype != q.dtype \
+                or pool_table.shape[-1] != page_table.shape[-1]:
+            raise KernelError("attention: the pooled cache must be shaped like the tokens'")
     if scale is None:
         scale = head_dim ** -0.5
     status = lib.ei_attention(
@@ -628,8 +660,32 @@ def attention(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items, row_
         None if slopes is None else _gpu(slopes, "slopes", torch.float32),
         None if sinks is None else _gpu(sinks, "sinks", torch.float32), float(scale), n_splits,
         key_heads, int(bool(values_in_keys)),
-        None if gate is None else _gpu(gate, "gate", torch.float32), _stream())
+        None if gate is None else _gpu(gate, "gate", torch.float32), int(pool or 0),
+        _gpu(pool_k, "pool_k") if pool else None, _gpu(pool_v, "pool_v") if pool else None,
+        _gpu(pool_table, "pool_table", torch.int32) if pool else None, _stream())
     _check(lib, status, "attention")
+
+
+def pool_store(k_pages, v_pages, row_pos, row_seq, page_table, pool_table, pool_k, pool_v, n_rows,
+               pool) -> None:
+    """For every row whose position ends a block of `pool` positions: the means of the block's
+    cached keys and values (all kv heads) into entry position // pool of the pooled cache."""
+    lib = library("attention_generic")
+    n_kv_heads, head_dim, value_dim = k_pages.shape[1], k_pages.shape[3], v_pages.shape[3]
+    if tuple(pool_k.shape[1:]) != tuple(k_pages.shape[1:]) or \
+            tuple(pool_v.shape[1:]) != tuple(v_pages.shape[1:]) or \
+            not (k_pages.dtype == v_pages.dtype == pool_k.dtype == pool_v.dtype) or \
+            pool_table.shape[-1] != page_table.shape[-1]:
+        raise KernelError("pool_store: the pooled cache must be shaped like the tokens'")
+    if row_pos.numel() < n_rows or row_seq.numel() < n_rows or pool < 1:
+        raise KernelError("pool_store: row metadata shorter than the rows")
+    status = lib.ei_pool_store(
+        _gpu(k_pages, "k_pages"), _gpu(v_pages, "v_pages"), _code(k_pages, "k_pages"),
+        _gpu(row_pos, "row_pos", torch.int32), _gpu(row_seq, "row_seq", torch.int32),
+        _gpu(page_table, "page_table", torch.int32), _gpu(pool_table, "pool_table", torch.int32),
+        page_table.shape[-1], _gpu(pool_k, "pool_k"), _gpu(pool_v, "pool_v"), n_rows, n_kv_heads,
+        head_dim, value_dim, int(pool), _stream())
+    _check(lib, status, "pool_store")
 
 
 def attention_wide_supported(dtype, query_width: int, head_dim: int, value_dim: int) -> bool:
@@ -908,8 +964,13 @@ def projection_norm_store(qkv, q_norm_w, k_norm_w, eps, row_pos, row_seq, page_t
 
 def head_store(proj, q_norm_w, k_norm_w, eps, frequencies, row_pos, row_seq, page_table, q_out,
                k_pages, v_pages, n_heads, n_kv_heads, head_dim, value_dim, write_cache=True,
-               v_first=None, v_mode=0, v_lambda=None) -> None:
-    """Rows that begin with [q | k | v] (and may go on with other columns), as [n, g] or float32
+               v_first=None, v_mode=0, v_lambda=None, query_temperature=None, gate_out=None,
+               gate_column=0) -> None:
+    """(query_temperature (coef, every): a query at position p is multiplied by
+    1 + coef ln(floor((p + 1) / every) + 1); gate_out float32 [n, heads]: receives the rows'
+    columns gate_column .. gate_column + heads - 1, summed over slices; n_kv_heads 0: the rows
+    hold queries only and the cache is not written.)
+    Rows that begin with [q | k | v] (and may go on with other columns), as [n, g] or float32
     slices [s, n, g]: per-head RMS norm of queries and keys (weights [head_dim], or None), the
     rotation of every head's first R elements in pairs (i, i + R/2) by position *
     frequencies[i] (float64 [R/2], or None for no rotation), queries to `q_out`, keys
@@ -947,6 +1008,14 @@ def head_store(proj, q_norm_w, k_norm_w, eps, frequencies, row_pos, row_seq, pag
         raise KernelError("head_store: v_first must be float32 [rows, kv heads * value_dim]")
     if v_mode == 2 and (v_lambda is None or v_lambda.numel() != 1):
         raise KernelError("head_store: mixing values needs its one weight")
+    temp = (0.0, 0) if query_temperature is None else query_temperature
+    if temp[1] < 0:
+        raise KernelError("head_store: the temperature's step must be positive")
+    if gate_out is not None and (tuple(gate_out.shape) != (n, n_heads)
+                                 or stride < gate_column + n_heads):
+        raise KernelError("head_store: gate_out must be [rows, heads] and the rows hold its columns")
+    if n_kv_heads == 0 and write_cache:
+        raise KernelError("head_store: rows without keys cannot write the cache")
     status = lib.ei_head_store(
         _gpu(proj, "proj"), _code(proj, "proj"), nsplit, split_stride, stride,
         None if q_norm_w is None else _gpu(q_norm_w, "q_norm", torch.float32),
@@ -958,7 +1027,9 @@ def head_store(proj, q_norm_w, k_norm_w, eps, frequencies, row_pos, row_seq, pag
         _gpu(v_pages, "v_pages") if write_cache else None, _code(q_out, "q_out"),
         None if not v_mode else _gpu(v_first, "v_first", torch.float32), int(v_mode),
         None if v_mode != 2 else _gpu(v_lambda, "v_lambda", torch.float32), n, n_heads,
-        n_kv_heads, head_dim, value_dim, int(write_cache), _stream())
+        n_kv_heads, head_dim, value_dim, int(write_cache), float(temp[0]), int(temp[1]),
+        None if gate_out is None else _gpu(gate_out, "gate_out", torch.float32), int(gate_column),
+        _stream())
     _check(lib, status, "head_store")
 
 
@@ -1383,11 +1454,170 @@ def ssm_out(y_raw, proj, norm_w, eps, shape: SsmShape, parts, row_seq, out) -> N
 
 
 # ---------------------------------------------------------------------------
-def moe_route(x, router_w, row_seq, expert, weight) -> None:
+def stream_norm(residual, delta, out, *, w_after=None, b_after=None, w_next=None, b_next=None,
+                eps: float, centred: bool, rows=None, write_residual: bool = True,
+                delta_bias=None) -> None:
+    """One pass over the rows of the float32 stream `residual` [R, H].  With d the sum of
+    delta's slices (+ delta_bias [H]): if `w_after` is given, d <- norm(d) * w_after + b_after
+    (the norm on a sublayer's output); residual += d (stored back unless told not to); if
+    `out` is given, out[i] = norm(residual[rows[i] if rows else i]) * w_next + b_next in out's
+    type.  centred: norms with a mean (layer norms; the biases may be None), else RMS norms.
+    delta None: nothing is added."""
+    lib = library("norms")
+    total_rows, hidden = residual.shape
+    n = total_rows if rows is None else rows.numel()
+    if out is not None and tuple(out.shape) != (n, hidden):
+        raise KernelError(f"stream_norm: out must be [{n}, {hidden}], got {list(out.shape)}")
+    if (out is None) != (w_next is None):
+        raise KernelError("stream_norm: an output and its norm's weight come together")
+    if delta is None and (w_after is not None or delta_bias is not None):
+        raise KernelError("stream_norm: a norm on a sublayer's output needs that output")
+    for name, vector in (("w_after", w_after), ("b_after", b_after), ("w_next", w_next),
+                         ("b_next", b_next), ("delta_bias", delta_bias)):
+        if vector is not None and vector.numel() != hidden:
+            raise KernelError(f"stream_norm: {name} must have {hidden} elements")
+    nsplit, stride, delta_ptr, delta_code = 0, 0, None, F32
+    if delta is not None:
+        nsplit, stride = _splits(delta, total_rows, hidden, "delta")
+        delta_ptr, delta_code = _gpu(delta, "delta"), _code(delta, "delta")
+
+    def f32(vector, name):
+        return None if vector is None else _gpu(vector, name, torch.float32)
+    status = lib.ei_stream_norm(
+        _gpu(residual, "residual", torch.float32), delta_ptr, delta_code, nsplit, stride,
+        f32(delta_bias, "delta_bias"), None if rows is None else _gpu(rows, "rows", torch.int32),
+        f32(w_after, "w_after"), f32(b_after, "b_after"), f32(w_next, "w_next"),
+        f32(b_next, "b_next"), float(eps), int(bool(centred)),
+        None if out is None else _gpu(out, "out"), F32 if out is None else _code(out, "out"), n,
+        hidden, int(write_residual), _stream())
+    _check(lib, status, "stream_norm")
+
+
+def norm_mean(branches, weights, eps: float, out: torch.Tensor) -> None:
+    """out [n, h] float32 = the mean over the branches b of rmsnorm(x_b) * w_b; every x_b is
+    [n, h] or float32 slices [s, n, h], of its own type."""
+    lib = library("norms")
+    rows, hidden = out.shape
+    count = len(branches)
+    if not 1 <= count <= 4 or len(weights) != count:
+        raise KernelError("norm_mean: 1 to 4 branches, each with its weight")
+    pointers = (c_void_p * count)()
+    weight_pointers = (c_void_p * count)()
+    nsplits = (c_int * count)()
+    strides = (c_longlong * count)()
+    codes = (c_int * count)()
+    for index, (x, w) in enumerate(zip(branches, weights)):
+        nsplits[index], strides[index] = _splits(x, rows, hidden, "a branch")
+        pointers[index] = _gpu(x, "a branch")
+        codes[index] = _code(x, "a branch")
+        if w.numel() != hidden:
+            raise KernelError(f"norm_mean: a weight must have {hidden} elements")
+        weight_pointers[index] = _gpu(w, "weight", torch.float32)
+    status = lib.ei_norm_mean(pointers, nsplits, strides, codes, weight_pointers, count,
+                              float(eps), _gpu(out, "out", torch.float32), rows, hidden, _stream())
+    _check(lib, status, "norm_mean")
+
+
+def input_conv(h, weight, state, part: int, parts: int, row_pos, row_seq, seq_in, seq_out,
+               seq_start, seq_count, seq_row0, out) -> None:
+    """out [n, w] = h + conv(h): a causal convolution over the rows of every sequence with
+    the filter weight [w, taps] (float32), the inputs before the step's rows taken from part
+    `part` of the sequence's state row (float32 rows of parts * (taps - 1) * w, two versions:
+    `seq_in` names the row read, `seq_out` the row whose part is written anew).  state None
+    with one tap."""
+    lib = library("input_conv")
+    n, width = h.shape
+    taps = weight.shape[1]
+    n_seqs = seq_count.numel()
+    if tuple(weight.shape) != (width, taps) or tuple(out.shape) != (n, width) or out.dtype != h.dtype:
+        raise KernelError("input_conv: shapes do not fit")
+    if out.data_ptr() == h.data_ptr():
+        raise KernelError("input_conv: the result needs a buffer of its own")
+    if taps > 1:
+        if state is None or state.dim() != 2 or state.shape[1] != parts * (taps - 1) * width:
+            raise KernelError("input_conv: state rows must hold parts * (taps - 1) * width floats")
+        if seq_in.numel() < n_seqs or seq_out.numel() < n_seqs:
+            raise KernelError("input_conv: state rows missing")
+    if row_pos.numel() < n or row_seq.numel() < n or seq_start.numel() < n_seqs \
+            or seq_row0.numel() < n_seqs:
+        raise KernelError("input_conv: row metadata shorter than the rows")
+    status = lib.ei_input_conv(
+        _gpu(h, "h"), _code(h, "h"), _gpu(weight, "weight", torch.float32),
+        None if taps == 1 else _gpu(state, "state", torch.float32), int(part), int(parts), taps,
+        _gpu(row_pos, "row_pos", torch.int32), _gpu(row_seq, "row_seq", torch.int32),
+        None if taps == 1 else _gpu(seq_in, "seq_in", torch.int32),
+        None if taps == 1 else _gpu(seq_out, "seq_out", torch.int32),
+        _gpu(seq_start, "seq_start", torch.int32), _gpu(seq_count, "seq_count", torch.int32),
+        _gpu(seq_row0, "seq_row0", torch.int32), _gpu(out, "out"), n, width, n_seqs, _stream())
+    _check(lib, status, "input_conv")
+
+
+def la_state_floats(heads: int, key_dim: int, value_dim: int) -> int:
+    """float32 elements of one sequence's linear-attention state: S [heads, key_dim, value_dim]."""
+    return heads * key_dim * value_dim
+
+
+def la_scan(proj, decay, state, seq_in, seq_out, seq_count, seq_row0, o_raw, heads, key_dim,
+            value_dim) -> None:
+    """The recurrence of linear attention with a decay per head over the rows of every
+    sequence: proj rows [q | k | v | ...] ([n, g] or float32 slices [s, n, g]), silu on all
+    three, S_t = decay_h S_(t-1) + k_t v_t^T, o_raw [n, heads * value_dim] float32 = S_t^T q_t.
+    state: float32 rows of heads * key_dim * value_dim, two versions (`seq_in`, `seq_out`)."""
+    lib = library("linear_attention")
+    n = o_raw.shape[0]
+    stride = proj.shape[-1]
+    nsplit, split_stride = _splits(proj, n, stride, "proj")
+    n_seqs = seq_count.numel()
+    if tuple(o_raw.shape) != (n, heads * value_dim) or decay.numel() != heads:
+        raise KernelError("la_scan: shapes do not fit")
+    if state.dim() != 2 or state.shape[1] != la_state_floats(heads, key_dim, value_dim):
+        raise KernelError("la_scan: state rows must hold heads * key_dim * value_dim floats")
+    if stride < heads * (2 * key_dim + value_dim):
+        raise KernelError("la_scan: the rows are narrower than q, k and v")
+    if seq_in.numel() < n_seqs or seq_out.numel() < n_seqs or seq_row0.numel() < n_seqs:
+        raise KernelError("la_scan: sequence metadata shorter than the sequences")
+    status = lib.ei_la_scan(
+        _gpu(proj, "proj"), _code(proj, "proj"), nsplit, split_stride, stride,
+        _gpu(decay, "decay", torch.float32), _gpu(state, "state", torch.float32),
+        _gpu(seq_in, "seq_in", torch.int32), _gpu(seq_out, "seq_out", torch.int32),
+        _gpu(seq_count, "seq_count", torch.int32), _gpu(seq_row0, "seq_row0", torch.int32),
+        _gpu(o_raw, "o_raw", torch.float32), n_seqs, heads, key_dim, value_dim, _stream())
+    _check(lib, status, "la_scan")
+
+
+def la_out(o_raw, proj, gate_column: int, norm_w, eps: float, row_seq, out) -> None:
+    """out [n, v] = rmsnorm(o_raw) * norm_w * sigmoid(g), g the columns gate_column ..
+    gate_column + v - 1 of proj's rows (summed over slices)."""
+    lib = library("linear_attention")
+    n, width = o_raw.shape
+    stride = proj.shape[-1]
+    nsplit, split_stride = _splits(proj, n, stride, "proj")
+    if tuple(out.shape) != (n, width) or norm_w.numel() != width or stride < gate_column + width:
+        raise KernelError("la_out: shapes do not fit")
+    status = lib.ei_la_out(
+        _gpu(o_raw, "o_raw", torch.float32), _gpu(proj, "proj"), _code(proj, "proj"), nsplit,
+        split_stride, stride, int(gate_column), _gpu(norm_w, "norm_w", torch.float32), float(eps),
+        None if row_seq is None else _gpu(row_seq, "row_seq", torch.int32), _gpu(out, "out"),
+        _code(out, "out"), n, width, _stream())
+    _check(lib, status, "la_out")
+
+
+ROUTER_SCORINGS = {"softmax_chosen": 0, "softmax_all": 1}
+
+
+def moe_route(x, router_w, row_seq, expert, weight, scoring: str = "softmax_chosen",
+              correction=None) -> None:
     """For every row of x [n, w]: the `top` experts of largest float32 logit router_w [E, w] . x
     into `expert` (int32 [n, top], largest first), the softmax over their logits into `weight`
-    (float32 [n, top]).  Rows with row_seq < 0 get weights of 0."""
+    (float32 [n, top]).  Rows with row_seq < 0 get weights of 0.  scoring "softmax_all": the
+    scores are the softmax over all E logits, the choice is by score + correction [E] (None:
+    by the score), and the weights are the chosen scores themselves."""
     lib = library("moe")
+    if scoring not in ROUTER_SCORINGS:
+        raise KernelError(f"moe_route: unknown scoring '{scoring}'")
+    if correction is not None and (scoring != "softmax_all" or correction.numel() != router_w.shape[0]):
+        raise KernelError("moe_route: a correction belongs to the scoring 'softmax_all' and has "
+                          "one number a router output")
     n, width = x.shape
     n_experts = router_w.shape[0]
     top = expert.shape[1]
@@ -1400,6 +1630,8 @@ def moe_route(x, router_w, row_seq, expert, weight) -> None:
                               None if row_seq is None else _gpu(row_seq, "row_seq", torch.int32),
                               _gpu(expert, "expert", torch.int32),
                               _gpu(weight, "weight", torch.float32), n, width, n_experts, top,
+                              ROUTER_SCORINGS[scoring],
+                              None if correction is None else _gpu(correction, "correction", torch.float32),
                               _stream())
     _check(lib, status, "moe_route")
 
@@ -1407,7 +1639,8 @@ def moe_route(x, router_w, row_seq, expert, weight) -> None:
 def moe_experts(x, w_gate, w_up, w_down, expert, weight, act, out) -> None:
     """out [n, w] float32 = sum over a row's choices k of weight[r, k] *
     w_down[e] (silu(w_gate[e] x_r) * (w_up[e] x_r)), e = expert[r, k]; w_gate and w_up
-    [E, f, w], w_down [E, w, f], all of x's type; `act` [n * top, f] of that type is scratch."""
+    [E, f, w], w_down [E, w, f], all of x's type; `act` [n * top, f] of that type is scratch.
+    A choice e >= E is an identity expert: it adds weight[r, k] * x_r."""
     lib = library("moe")
     n, width = x.shape
     n_experts, inter = w_gate.shape[0], w_gate.shape[1]
@@ -1424,7 +1657,8 @@ def moe_experts(x, w_gate, w_up, w_down, expert, weight, act, out) -> None:
                                 _gpu(w_down, "w_down"), _code(x, "x"),
                                 _gpu(expert, "expert", torch.int32),
                                 _gpu(weight, "weight", torch.float32), _gpu(act, "act"),
-                                _gpu(out, "out", torch.float32), n, width, inter, top, _stream())
+                                _gpu(out, "out", torch.float32), n, width, inter, n_experts, top,
+                                _stream())
     _check(lib, status, "moe_experts")
 
 

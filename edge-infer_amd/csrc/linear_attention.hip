@@ -1,0 +1,210 @@
+// Linear attention with a fixed decay per head.  A row of the projection is
+// [q: H * DK | k: H * DK | v: H * DV | g: H * DV]; with q, k, v passed through silu, per head
+//
+//   S_t = decay_h S_(t-1) + k_t v_t^T        S is [DK, DV], float32, zero before the sequence
+//   o_t = S_t^T q_t
+//
+// and then out = rmsnorm(o over all heads) * w * sigmoid(g) in the rows' type.  The state is a
+// float32 table with two versions of every sequence's row ([H][DK][DV]): a step reads the row
+// `seq_in` names and writes the whole row `seq_out` names.  The walk over a sequence's tokens
+// is a true recurrence: tokens are taken in order, one after the other, whatever the step
+// holds (a whole prompt, a portion, one token), so a position's result does not depend on how
+// its sequence was cut.
+#include "common.h"
+
+namespace {
+
+constexpr int kTile = 16;      // tokens whose operands lie in LDS at a time
+constexpr int kCols = 64;      // columns of S a block owns
+constexpr int kGroups = 4;     // waves of a block: each owns a quarter of the rows of S
+
+template <typename TI>
+__device__ __forceinline__ float sliced(const TI* p, int nsplit, size_t split_stride) {
+  float v = 0.f;
+  for (int s = 0; s < nsplit; ++s) v += ei::to_f32<TI>(p[s * split_stride]);
+  return v;
+}
+
+__device__ __forceinline__ float silu_f32(float x) { return x / (1.0f + expf(-x)); }
+
+// A block a (sequence, head, 64 columns of S).  Thread (c, g): column c, rows g R .. g R + R - 1
+// (R a multiple of 4, kGroups * R >= DK; rows beyond DK hold zeros).
+template <typename TI, int R>
+__global__ void __launch_bounds__(kCols * kGroups)
+la_scan_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride, size_t row_stride,
+               const float* __restrict__ decay, const float* state_in_table, float* state_out_table,
+               const int32_t* __restrict__ seq_in, const int32_t* __restrict__ seq_out,
+               const int32_t* __restrict__ seq_count, const int32_t* __restrict__ seq_row0,
+               float* __restrict__ o_raw, int H, int DK, int DV) {
+  constexpr int DKP = kGroups * R;
+  __shared__ __attribute__((aligned(16))) float qs[kTile][DKP];
+  __shared__ __attribute__((aligned(16))) float ks[kTile][DKP];
+  __shared__ float vs[kTile][kCols];
+  __shared__ float part[kTile][kGroups][kCols];
+  const int seq = blockIdx.x, head = blockIdx.y, col0 = blockIdx.z * kCols;
+  const int count = seq_count[seq];
+  if (count <= 0) return;                       // a padding sequence
+  const int t = threadIdx.x, c = t % kCols, g = t / kCols;
+  const int col = col0 + c;
+  const bool col_live = col < DV;
+  const size_t state_floats = static_cast<size_t>(H) * DK * DV;
+  const float* s_in = state_in_table + static_cast<size_t>(seq_in[seq]) * state_floats +
+                      static_cast<size_t>(head) * DK * DV;
+  float* s_out = state_out_table + static_cast<size_t>(seq_out[seq]) * state_floats +
+                 static_cast<size_t>(head) * DK * DV;
+  float S[R];
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    const int row = g * R + i;
+    S[i] = (col_live && row < DK) ? s_in[static_cast<size_t>(row) * DV + col] : 0.f;
+  }
+  const float d = decay[head];
+  const int row0 = seq_row0[seq];
+  const size_t q_at = static_cast<size_t>(head) * DK;
+  const size_t k_at = static_cast<size_t>(H) * DK + q_at;
+  const size_t v_at = 2 * static_cast<size_t>(H) * DK + static_cast<size_t>(head) * DV + col0;
+  const size_t out_width = static_cast<size_t>(H) * DV;
+
+  for (int tile0 = 0; tile0 < count; tile0 += kTile) {
+    const int nt = min(kTile, count - tile0);
+    for (int idx = t; idx < nt * DKP; idx += kCols * kGroups) {
+      const int tt = idx / DKP, row = idx % DKP;
+      float qv = 0.f, kv = 0.f;
+      if (row < DK) {
+        const TI* src = proj + static_cast<size_t>(row0 + tile0 + tt) * row_stride;
+        qv = silu_f32(sliced(src + q_at + row, nsplit, split_stride));
+        kv = silu_f32(sliced(src + k_at + row, nsplit, split_stride));
+      }
+      qs[tt][row] = qv;
+      ks[tt][row] = kv;
+    }
+    for (int idx = t; idx < nt * kCols; idx += kCols * kGroups) {
+      const int tt = idx / kCols, cc = idx % kCols;
+      float vv = 0.f;
+      if (col0 + cc < DV)
+        vv = silu_f32(sliced(proj + static_cast<size_t>(row0 + tile0 + tt) * row_stride + v_at + cc,
+                             nsplit, split_stride));
+      vs[tt][cc] = vv;
+    }
+    __syncthreads();
+    for (int tt = 0; tt < nt; ++tt) {
+      const float vv = vs[tt][c];
+      const float4* kq = reinterpret_cast<const float4*>(&ks[tt][g * R]);
+      const float4* qq = reinterpret_cast<const float4*>(&qs[tt][g * R]);
+      float acc = 0.f;
+#pragma unroll
+      for (int i4 = 0; i4 < R / 4; ++i4) {
+        const float4 k4 = kq[i4], q4 = qq[i4];
+        S[4 * i4 + 0] = d * S[4 * i4 + 0] + k4.x * vv;
+        S[4 * i4 + 1] = d * S[4 * i4 + 1] + k4.y * vv;
+        S[4 * i4 + 2] = d * S[4 * i4 + 2] + k4.z * vv;
+        S[4 * i4 + 3] = d * S[4 * i4 + 3] + k4.w * vv;
+        acc += S[4 * i4 + 0] * q4.x;
+        acc += S[4 * i4 + 1] * q4.y;
+        acc += S[4 * i4 + 2] * q4.z;
+        acc += S[4 * i4 + 3] * q4.w;
+      }
+      part[tt][g][c] = acc;
+    }
+    __syncthreads();
+    for (int idx = t; idx < nt * kCols; idx += kCols * kGroups) {
+      const int tt = idx / kCols, cc = idx % kCols;
+      if (col0 + cc < DV) {
+        float o = part[tt][0][cc];
+#pragma unroll
+        for (int gg = 1; gg < kGroups; ++gg) o += part[tt][gg][cc];
+        o_raw[static_cast<size_t>(row0 + tile0 + tt) * out_width + static_cast<size_t>(head) * DV +
+              col0 + cc] = o;
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    const int row = g * R + i;
+    if (col_live && row < DK) s_out[static_cast<size_t>(row) * DV + col] = S[i];
+  }
+}
+
+// A block a row: out = o / sqrt(mean(o^2) + eps) * w * sigmoid(g), g the columns of the
+// projection from `gate_at` on (the sum of its float32 slices).
+template <typename TI, typename TO>
+__global__ void la_out_kernel(const float* __restrict__ o_raw, const TI* __restrict__ proj, int nsplit,
+                              size_t split_stride, size_t row_stride, size_t gate_at,
+                              const float* __restrict__ norm_w, float eps,
+                              const int32_t* __restrict__ row_seq, TO* __restrict__ out, int HV) {
+  __shared__ float scratch[16];
+  const int row = blockIdx.x;
+  if (row_seq && row_seq[row] < 0) return;      // a padding row
+  const float* o = o_raw + static_cast<size_t>(row) * HV;
+  float squares = 0.f;
+  for (int i = threadIdx.x; i < HV; i += blockDim.x) squares += o[i] * o[i];
+  const float inv = 1.0f / sqrtf(ei::block_sum(squares, scratch) / static_cast<float>(HV) + eps);
+  const TI* gate = proj + static_cast<size_t>(row) * row_stride + gate_at;
+  for (int i = threadIdx.x; i < HV; i += blockDim.x) {
+    const float gv = sliced(gate + i, nsplit, split_stride);
+    const float y = (o[i] * inv) * norm_w[i] / (1.0f + expf(-gv));
+    out[static_cast<size_t>(row) * HV + i] = ei::from_f32<TO>(y);
+  }
+}
+
+}  // namespace
+
+// Floats of one sequence's state.
+extern "C" long long ei_la_state_floats(int H, int DK, int DV) {
+  return static_cast<long long>(H) * DK * DV;
+}
+
+// proj: [nsplit][N, row_stride] of proj_dtype, rows as above; state: float32 rows of
+// H * DK * DV; o_raw: float32 [N, H * DV].
+extern "C" int ei_la_scan(const void* proj, int proj_dtype, int nsplit, long long split_stride,
+                          long long row_stride, const float* decay, float* state,
+                          const int32_t* seq_in, const int32_t* seq_out, const int32_t* seq_count,
+                          const int32_t* seq_row0, float* o_raw, int n_seqs, int H, int DK, int DV,
+                          hipStream_t stream) {
+  EI_REQUIRE(proj && decay && state && seq_in && seq_out && seq_count && seq_row0 && o_raw,
+             "la_scan: null pointer");
+  EI_REQUIRE(n_seqs > 0 && H > 0 && DK >= 1 && DK <= 256 && DV >= 1 && nsplit >= 1,
+             "la_scan: key heads of 1 to 256 elements");
+  EI_REQUIRE(row_stride >= 2LL * H * DK + 1LL * H * DV, "la_scan: rows narrower than q, k and v");
+  EI_REQUIRE(H <= 65535 && (DV + kCols - 1) / kCols <= 65535, "la_scan: too many heads");
+  const dim3 grid(n_seqs, H, (DV + kCols - 1) / kCols);
+  const size_t ss = static_cast<size_t>(split_stride), rs = static_cast<size_t>(row_stride);
+#define EI_LA(TI, R)                                                                           \
+  la_scan_kernel<TI, R><<<grid, kCols * kGroups, 0, stream>>>(                                 \
+      static_cast<const TI*>(proj), nsplit, ss, rs, decay, state, state, seq_in, seq_out,      \
+      seq_count, seq_row0, o_raw, H, DK, DV)
+#define EI_LA_T(TI)                                 \
+  do {                                              \
+    if (DK <= 32) EI_LA(TI, 8);                     \
+    else if (DK <= 64) EI_LA(TI, 16);               \
+    else if (DK <= 128) EI_LA(TI, 32);              \
+    else EI_LA(TI, 64);                             \
+  } while (0)
+  if (proj_dtype == EI_F32) EI_LA_T(float);
+  else if (proj_dtype == EI_BF16) EI_LA_T(bf16_t);
+  else EI_REQUIRE(false, "la_scan: unknown dtype");
+#undef EI_LA_T
+#undef EI_LA
+  EI_LAUNCH_CHECK();
+}
+
+extern "C" int ei_la_out(const float* o_raw, const void* proj, int proj_dtype, int nsplit,
+                         long long split_stride, long long row_stride, long long gate_at,
+                         const float* norm_w, float eps, const int32_t* row_seq, void* out,
+                         int out_dtype, int N, int HV, hipStream_t stream) {
+  EI_REQUIRE(o_raw && proj && norm_w && out && N > 0 && HV > 0 && nsplit >= 1, "la_out: bad arguments");
+  EI_REQUIRE(row_stride >= gate_at + HV, "la_out: rows narrower than the gate's columns");
+  const int threads = HV >= 2048 ? 512 : (HV >= 512 ? 256 : 128);
+  const size_t ss = static_cast<size_t>(split_stride), rs = static_cast<size_t>(row_stride);
+  const size_t ga = static_cast<size_t>(gate_at);
+#define EI_LO(TI, TO)                                                                          \
+  la_out_kernel<TI, TO><<<N, threads, 0, stream>>>(o_raw, static_cast<const TI*>(proj), nsplit, ss, \
+                                                   rs, ga, norm_w, eps, row_seq,               \
+                                                   static_cast<TO*>(out), HV)
+  if (proj_dtype == EI_F32 && out_dtype == EI_F32) EI_LO(float, float);
+  else if (proj_dtype == EI_F32 && out_dtype == EI_BF16) EI_LO(float, bf16_t);
+  else if (proj_dtype == EI_BF16 && out_dtype == EI_BF16) EI_LO(bf16_t, bf16_t);
+  else EI_REQUIRE(false, "la_out: unsupported dtype combination");
+#undef EI_LO
+  EI_LAUNCH_CHECK();
+}

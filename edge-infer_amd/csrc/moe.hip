@@ -2,8 +2,12 @@
 //
 // Router: logits z = W_router x in float32 (W_router is kept in float32; x is read as stored),
 // the `top` experts of largest logit (of equal logits the one of lower index), and their
-// weights softmax(z over the chosen ones only).  Experts: for row r and its choice k with expert
-// e and weight p,  y_r += p W_down,e (silu(W_gate,e x_r) * (W_up,e x_r)).
+// weights softmax(z over the chosen ones only); or (`mode` 1) the scores s = softmax(z) over all
+// router outputs, the `top` outputs of largest s + correction (a learned number per output,
+// null: none), and the weights s of the chosen, not renormalised.  Experts: for row r and its
+// choice k with expert e and weight p,  y_r += p W_down,e (silu(W_gate,e x_r) * (W_up,e x_r)).
+// A router may have more outputs than there are experts: an output beyond the experts is an
+// identity expert, which adds p x_r and has no matrices.
 //
 // Two forms of the experts.  One takes a (row, choice) pair at a time and streams the expert's
 // matrices for it: any type and any sizes.  The other (bfloat16, widths that are multiples of
@@ -23,7 +27,8 @@ template <typename TX>
 __global__ void __launch_bounds__(256)
 moe_route_kernel(const TX* __restrict__ x, const float* __restrict__ w_router,
                  const int32_t* __restrict__ row_seq, int32_t* __restrict__ expert,
-                 float* __restrict__ weight, int N, int W, int E, int top) {
+                 float* __restrict__ weight, int N, int W, int E, int top, int mode,
+                 const float* __restrict__ correction) {
   __shared__ float logits[kRouteMax * EI_WAVE];
   const int wave = threadIdx.x / EI_WAVE, lane = threadIdx.x % EI_WAVE;
   const int row = blockIdx.x;
@@ -60,6 +65,27 @@ moe_route_kernel(const TX* __restrict__ x, const float* __restrict__ w_router,
   float z[kRouteMax];
 #pragma unroll
   for (int j = 0; j < kRouteMax; ++j) z[j] = lane + j * EI_WAVE < E ? logits[lane + j * EI_WAVE] : -FLT_MAX;
+  float score[kRouteMax];                        // mode 1: the softmax over all outputs
+  if (mode == 1) {
+    float top_z = -FLT_MAX;
+#pragma unroll
+    for (int j = 0; j < kRouteMax; ++j) top_z = fmaxf(top_z, z[j]);
+    top_z = ei::wave_max(top_z);
+    float sum = 0.f;
+#pragma unroll
+    for (int j = 0; j < kRouteMax; ++j) {
+      score[j] = lane + j * EI_WAVE < E ? expf(z[j] - top_z) : 0.f;
+      sum += score[j];
+    }
+    sum = ei::wave_sum(sum);
+#pragma unroll
+    for (int j = 0; j < kRouteMax; ++j) {
+      const int e = lane + j * EI_WAVE;
+      score[j] = score[j] / sum;
+      // what the choice goes by from here on
+      z[j] = e < E ? score[j] + (correction ? correction[e] : 0.f) : -FLT_MAX;
+    }
+  }
   unsigned taken = 0;                            // bit j: this lane's expert lane + 64 j is chosen
   float total = 0.f, largest = 0.f;
   float mine = 0.f;                              // lane k keeps the k-th choice
@@ -77,14 +103,23 @@ moe_route_kernel(const TX* __restrict__ x, const float* __restrict__ w_router,
       const int other_e = __shfl_xor(best_e, offset, EI_WAVE);
       if (other > best || (other == best && other_e < best_e)) { best = other; best_e = other_e; }
     }
-    if (best_e % EI_WAVE == lane) taken |= 1u << (best_e / EI_WAVE);
+    float chosen_score = 0.f;                    // mode 1: the score of the choice, from its lane
+    if (best_e % EI_WAVE == lane) {
+      taken |= 1u << (best_e / EI_WAVE);
+      if (mode == 1) {
+#pragma unroll
+        for (int j = 0; j < kRouteMax; ++j)
+          if (j == best_e / EI_WAVE) chosen_score = score[j];
+      }
+    }
+    if (mode == 1) chosen_score = __shfl(chosen_score, best_e % EI_WAVE, EI_WAVE);
     if (k == 0) largest = best;
     total += expf(best - largest);
-    if (lane == k) { mine = best; mine_e = best_e; }
+    if (lane == k) { mine = mode == 1 ? chosen_score : best; mine_e = best_e; }
   }
   if (lane < top) {
     e_out[lane] = mine_e;
-    w_out[lane] = expf(mine - largest) / total;
+    w_out[lane] = mode == 1 ? mine : expf(mine - largest) / total;
   }
 }
 
@@ -94,10 +129,11 @@ template <typename T>
 __global__ void __launch_bounds__(256)
 moe_gate_up_kernel(const T* __restrict__ x, const T* __restrict__ w_gate, const T* __restrict__ w_up,
                    const int32_t* __restrict__ expert, const float* __restrict__ weight,
-                   T* __restrict__ act, int W, int F, int top) {
+                   T* __restrict__ act, int W, int F, int top, int E) {
   const int pair = blockIdx.x;
   if (weight[pair] == 0.f) return;              // a padding row's choice
   const int row = pair / top, e = expert[pair];
+  if (e >= E) return;                           // an identity expert has no product
   const int wave = threadIdx.x / EI_WAVE, lane = threadIdx.x % EI_WAVE;
   const int f0 = blockIdx.y * 16 + wave * 4;
   if (f0 >= F) return;
@@ -144,7 +180,7 @@ template <typename T>
 __global__ void __launch_bounds__(256)
 moe_down_kernel(const T* __restrict__ act, const T* __restrict__ w_down,
                 const int32_t* __restrict__ expert, const float* __restrict__ weight,
-                float* __restrict__ out, int W, int F, int top) {
+                float* __restrict__ out, int W, int F, int top, int E, const T* __restrict__ x) {
   const int row = blockIdx.x;
   const int wave = threadIdx.x / EI_WAVE, lane = threadIdx.x % EI_WAVE;
   const int c0 = blockIdx.y * 16 + wave * 4;
@@ -155,6 +191,11 @@ moe_down_kernel(const T* __restrict__ act, const T* __restrict__ w_down,
     const int pair = row * top + k;
     const float p = weight[pair];
     if (p == 0.f) continue;
+    if (expert[pair] >= E) {                    // an identity expert: the row itself
+      for (int q = 0; q < nc; ++q)
+        total[q] += p * ei::to_f32<T>(x[static_cast<size_t>(row) * W + c0 + q]);
+      continue;
+    }
     const T* a = act + static_cast<size_t>(pair) * F;
     const T* d = w_down + (static_cast<size_t>(expert[pair]) * W + c0) * F;
     float s[4] = {0.f, 0.f, 0.f, 0.f};
@@ -191,7 +232,8 @@ moe_down_kernel(const T* __restrict__ act, const T* __restrict__ w_down,
 //
 // moe_group: the (row, choice) pairs counted and laid out by expert: `sorted` [P] holds the
 // pairs of expert 0, then those of expert 1, ...; `place` [P] is where a pair went (-1: a pair
-// of weight 0, which is left out); `starts` [E + 1] are the experts' first places.  Which place
+// of weight 0, which is left out; -2: a pair of an identity expert, an output of the router
+// beyond the E experts); `starts` [E + 1] are the experts' first places.  Which place
 // a pair gets inside its expert's span depends on the order of the atomics; every pair is
 // computed for itself, so no result depends on it.
 __global__ void __launch_bounds__(1024)
@@ -202,7 +244,7 @@ moe_group_kernel(const int32_t* __restrict__ expert, const float* __restrict__ w
   for (int e = threadIdx.x; e < E; e += blockDim.x) counts[e] = 0;
   __syncthreads();
   for (int p = threadIdx.x; p < P; p += blockDim.x)
-    if (weight[p] != 0.f) atomicAdd(&counts[expert[p]], 1);
+    if (weight[p] != 0.f && expert[p] < E) atomicAdd(&counts[expert[p]], 1);
   __syncthreads();
   if (threadIdx.x == 0) {
     int at = 0;
@@ -217,8 +259,12 @@ moe_group_kernel(const int32_t* __restrict__ expert, const float* __restrict__ w
   for (int p = threadIdx.x; p < P; p += blockDim.x) {
     int q = -1;
     if (weight[p] != 0.f) {
-      q = atomicAdd(&cursor[expert[p]], 1);
-      sorted[q] = p;
+      if (expert[p] < E) {
+        q = atomicAdd(&cursor[expert[p]], 1);
+        sorted[q] = p;
+      } else {
+        q = -2;
+      }
     }
     place[p] = q;
   }
@@ -349,7 +395,7 @@ moe_gemm_kernel(const bf16_t* __restrict__ a, const int32_t* __restrict__ sorted
 // out [rows, W] = sum over a row's choices of weight * the choice's product row.
 __global__ void moe_combine_kernel(const float* __restrict__ sums, const int32_t* __restrict__ place,
                                    const float* __restrict__ weight, float* __restrict__ out,
-                                   int W, int top, size_t total) {
+                                   int W, int top, size_t total, const bf16_t* __restrict__ x) {
   const size_t start = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   const size_t step = static_cast<size_t>(gridDim.x) * blockDim.x;
   for (size_t idx = start; idx < total; idx += step) {
@@ -358,6 +404,7 @@ __global__ void moe_combine_kernel(const float* __restrict__ sums, const int32_t
     for (int k = 0; k < top; ++k) {
       const int q = place[row * top + k];
       if (q >= 0) sum += weight[row * top + k] * sums[static_cast<size_t>(q) * W + col];
+      else if (q == -2) sum += weight[row * top + k] * ei::bf16_to_f32(x[idx]);   // identity
     }
     out[idx] = sum;
   }
@@ -367,18 +414,21 @@ __global__ void moe_combine_kernel(const float* __restrict__ sums, const int32_t
 
 extern "C" int ei_moe_route(const void* x, int x_dtype, const float* w_router, const int32_t* row_seq,
                             int32_t* expert, float* weight, int N, int W, int E, int top,
-                            hipStream_t stream) {
+                            int mode, const float* correction, hipStream_t stream) {
   EI_REQUIRE(x && w_router && expert && weight && N > 0 && W > 0, "moe_route: bad arguments");
   EI_REQUIRE(E >= 1 && E <= kRouteMax * EI_WAVE && top >= 1 && top <= E && top <= kMaxTop,
              "moe_route: up to 512 experts, of which 1 to 64 are chosen");
+  EI_REQUIRE(mode == 0 || mode == 1, "moe_route: unknown mode");
   const int threads = 256;
   const unsigned blocks = static_cast<unsigned>(N);
   if (x_dtype == EI_F32)
     moe_route_kernel<float><<<blocks, threads, 0, stream>>>(static_cast<const float*>(x), w_router,
-                                                            row_seq, expert, weight, N, W, E, top);
+                                                            row_seq, expert, weight, N, W, E, top,
+                                                            mode, correction);
   else if (x_dtype == EI_BF16)
     moe_route_kernel<bf16_t><<<blocks, threads, 0, stream>>>(static_cast<const bf16_t*>(x), w_router,
-                                                             row_seq, expert, weight, N, W, E, top);
+                                                             row_seq, expert, weight, N, W, E, top,
+                                                            mode, correction);
   else
     EI_REQUIRE(false, "moe_route: unknown dtype");
   EI_LAUNCH_CHECK();
@@ -386,7 +436,7 @@ extern "C" int ei_moe_route(const void* x, int x_dtype, const float* w_router, c
 
 extern "C" int ei_moe_experts(const void* x, const void* w_gate, const void* w_up, const void* w_down,
                               int dtype, const int32_t* expert, const float* weight, void* act,
-                              float* out, int N, int W, int F, int top, hipStream_t stream) {
+                              float* out, int N, int W, int F, int E, int top, hipStream_t stream) {
   EI_REQUIRE(x && w_gate && w_up && w_down && expert && weight && act && out, "moe_experts: null pointer");
   EI_REQUIRE(N > 0 && W > 0 && F > 0 && top >= 1, "moe_experts: sizes must be positive");
   EI_REQUIRE(static_cast<long long>(N) * top <= 0x7fffffffLL && (F + 15) / 16 <= 65535 &&
@@ -396,9 +446,10 @@ extern "C" int ei_moe_experts(const void* x, const void* w_gate, const void* w_u
   do {                                                                                         \
     moe_gate_up_kernel<T><<<grid_up, 256, 0, stream>>>(                                        \
         static_cast<const T*>(x), static_cast<const T*>(w_gate), static_cast<const T*>(w_up),  \
-        expert, weight, static_cast<T*>(act), W, F, top);                                      \
+        expert, weight, static_cast<T*>(act), W, F, top, E);                                   \
     moe_down_kernel<T><<<grid_down, 256, 0, stream>>>(                                         \
-        static_cast<const T*>(act), static_cast<const T*>(w_down), expert, weight, out, W, F, top); \
+        static_cast<const T*>(act), static_cast<const T*>(w_down), expert, weight, out, W, F, top, \
+        E, static_cast<const T*>(x));                                                          \
   } while (0)
   if (dtype == EI_F32) EI_MOE(float);
   else if (dtype == EI_BF16) EI_MOE(bf16_t);
@@ -457,6 +508,6 @@ extern "C" int ei_moe_experts_grouped(const void* x, const void* w_gate, const v
   const size_t total = static_cast<size_t>(N) * W;
   size_t blocks = (total + 255) / 256;
   if (blocks > static_cast<size_t>(ei_compute_units()) * 16) blocks = static_cast<size_t>(ei_compute_units()) * 16;
-  moe_combine_kernel<<<static_cast<unsigned>(blocks), 256, 0, stream>>>(sums, place, weight, out, W, top, total);
+  moe_combine_kernel<<<static_cast<unsigned>(blocks), 256, 0, stream>>>(sums, place, weight, out, W, top, total, xb);
   EI_LAUNCH_CHECK();
 }

@@ -627,6 +627,10 @@ extern "C" int ei_projection_norm_store(
 // elements in pairs (i, i + R/2), then queries to q_out and keys to their page.  Value heads:
 // v_mode 0: stored as they are; 1: also written, in float32, to v_first [N, nkv * DV];
 // 2: v <- (1 - lambda) v + lambda v_first before the store (lambda one float on the device).
+// temp_every > 0: a query at position p is multiplied by 1 + temp_coef ln(p' + 1), p' the whole
+// part of (p + 1) / temp_every.  gate_out: the float32 sums of the nq columns from `gate_at` on
+// (one number a query head) go to gate_out [N, nq] for the attention kernel's output gate.
+// nkv may be 0 for rows that hold queries only (a layer that reads another layer's keys).
 namespace {
 
 constexpr int kHeadStoreMax = 8;  // elements a lane: head sizes up to 512
@@ -646,7 +650,8 @@ __global__ void head_store_kernel(
     const int32_t* __restrict__ row_seq, const int32_t* __restrict__ page_table, int table_width,
     TO* __restrict__ q_out, TO* __restrict__ k_pages, TO* __restrict__ v_pages,
     float* __restrict__ v_first, int v_mode, const float* __restrict__ v_lambda,
-    int N, int nq, int nkv, int D, int DV, int write_cache) {
+    int N, int nq, int nkv, int D, int DV, int write_cache, float temp_coef, int temp_every,
+    float* __restrict__ gate_out, size_t gate_at) {
   const int heads = nq + 2 * nkv;
   const int wave = (blockIdx.x * blockDim.x + threadIdx.x) / EI_WAVE;
   const int lane = threadIdx.x % EI_WAVE;
@@ -696,6 +701,10 @@ __global__ void head_store_kernel(
   }
   float inv = 1.0f;
   if (w) inv = 1.0f / sqrtf(ei::wave_sum(sum) / static_cast<float>(D) + eps);
+  const float warm = (is_q && temp_every > 0)
+      ? 1.0f + temp_coef * logf(static_cast<float>((pos + 1) / temp_every) + 1.0f) : 1.0f;
+  if (is_q && gate_out && lane == 0)
+    gate_out[static_cast<size_t>(row) * nq + head] = sliced(src_row + gate_at + head, nsplit, split_stride);
   TO* dst = is_q ? q_out + (static_cast<size_t>(row) * nq + head) * D
                  : k_pages + ((page_slot * nkv + (head - nq)) * EI_PAGE + pos % EI_PAGE) * static_cast<size_t>(D);
 #pragma unroll
@@ -713,7 +722,7 @@ __global__ void head_store_kernel(
       sincosf(angle, &sn, &cs);
       v = e < rhalf ? v * cs - p * sn : v * cs + p * sn;
     }
-    dst[e] = ei::from_f32<TO>(v);
+    dst[e] = ei::from_f32<TO>(v * warm);
   }
 }
 
@@ -741,7 +750,8 @@ __global__ void head_store_vec_kernel(
     const int32_t* __restrict__ row_seq, const int32_t* __restrict__ page_table, int table_width,
     TO* __restrict__ q_out, TO* __restrict__ k_pages, TO* __restrict__ v_pages,
     float* __restrict__ v_first, int v_mode, const float* __restrict__ v_lambda,
-    int N, int nq, int nkv, int D, int DV, int write_cache, int G) {
+    int N, int nq, int nkv, int D, int DV, int write_cache, int G, float temp_coef, int temp_every,
+    float* __restrict__ gate_out, size_t gate_at) {
   const int heads = nq + 2 * nkv;
   const size_t thread = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   const size_t item = thread / G;
@@ -821,6 +831,13 @@ __global__ void head_store_vec_kernel(
       x[i] = e0 < rhalf ? x[i] * cs - y[i] * sn : x[i] * cs + y[i] * sn;
     }
   }
+  if (is_q && temp_every > 0) {
+    const float warm = 1.0f + temp_coef * logf(static_cast<float>((pos + 1) / temp_every) + 1.0f);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) x[i] *= warm;
+  }
+  if (is_q && gate_out && j == 0)
+    gate_out[static_cast<size_t>(row) * nq + head] = sliced(src_row + gate_at + head, nsplit, split_stride);
   TO* dst = is_q ? q_out + (static_cast<size_t>(row) * nq + head) * D
                  : k_pages + ((page * nkv + (head - nq)) * EI_PAGE + pos % EI_PAGE) * static_cast<size_t>(D);
   ei::VecN<TO, 8>::store(dst + e0, x);
@@ -834,8 +851,12 @@ extern "C" int ei_head_store(
     const int32_t* row_pos, const int32_t* row_seq, const int32_t* page_table, int table_width,
     void* q_out, void* k_pages, void* v_pages, int out_dtype, float* v_first, int v_mode,
     const float* v_lambda, int N, int nq, int nkv, int D, int DV, int write_cache,
-    hipStream_t stream) {
-  EI_REQUIRE(N > 0 && nq > 0 && nkv > 0 && D > 0 && DV > 0, "head_store: sizes must be positive");
+    float temp_coef, int temp_every, float* gate_out, long long gate_at, hipStream_t stream) {
+  EI_REQUIRE(N > 0 && nq > 0 && nkv >= 0 && D > 0 && DV > 0, "head_store: sizes must be positive");
+  EI_REQUIRE(nkv > 0 || !write_cache, "head_store: rows without keys cannot write the cache");
+  EI_REQUIRE(temp_every >= 0, "head_store: negative temperature step");
+  EI_REQUIRE(!gate_out || (gate_at >= 0 && row_stride >= gate_at + nq),
+             "head_store: rows narrower than the gate's columns");
   EI_REQUIRE(D <= kHeadStoreMax * EI_WAVE, "head_store: head_dim above 512");
   EI_REQUIRE(proj && row_pos && row_seq && q_out && nsplit >= 1, "head_store: bad arguments");
   EI_REQUIRE(row_stride >= static_cast<long long>(nq + nkv) * D + static_cast<long long>(nkv) * DV,
@@ -866,7 +887,8 @@ extern "C" int ei_head_store(
   head_store_vec_kernel<TI, TO><<<vblocks, threads, 0, stream>>>(                              \
       static_cast<const TI*>(proj), nsplit, ss, rs, q_norm_w, k_norm_w, eps, freqs, R, row_pos, \
       row_seq, page_table, table_width, static_cast<TO*>(q_out), static_cast<TO*>(k_pages),    \
-      static_cast<TO*>(v_pages), v_first, v_mode, v_lambda, N, nq, nkv, D, DV, write_cache, G)
+      static_cast<TO*>(v_pages), v_first, v_mode, v_lambda, N, nq, nkv, D, DV, write_cache, G,  \
+      temp_coef, temp_every, gate_out, static_cast<size_t>(gate_at))
     if (in_dtype == EI_F32 && out_dtype == EI_F32) EI_HSV(float, float);
     else if (in_dtype == EI_F32 && out_dtype == EI_BF16) EI_HSV(float, bf16_t);
     else if (in_dtype == EI_BF16 && out_dtype == EI_BF16) EI_HSV(bf16_t, bf16_t);
@@ -878,7 +900,8 @@ extern "C" int ei_head_store(
   head_store_kernel<TI, TO><<<blocks, threads, 0, stream>>>(                                   \
       static_cast<const TI*>(proj), nsplit, ss, rs, q_norm_w, k_norm_w, eps, freqs, R, row_pos, \
       row_seq, page_table, table_width, static_cast<TO*>(q_out), static_cast<TO*>(k_pages),    \
-      static_cast<TO*>(v_pages), v_first, v_mode, v_lambda, N, nq, nkv, D, DV, write_cache)
+      static_cast<TO*>(v_pages), v_first, v_mode, v_lambda, N, nq, nkv, D, DV, write_cache,     \
+      temp_coef, temp_every, gate_out, static_cast<size_t>(gate_at))
   if (in_dtype == EI_F32 && out_dtype == EI_F32) EI_HS(float, float);
   else if (in_dtype == EI_F32 && out_dtype == EI_BF16) EI_HS(float, bf16_t);
   else if (in_dtype == EI_BF16 && out_dtype == EI_BF16) EI_HS(bf16_t, bf16_t);

@@ -152,9 +152,11 @@ class DecoderModel:
             self.layers.append(block_cls(layer, spec.hidden_size, own, self.dtype, self.device,
                                          positions=self.position_table))
         final_cls = lookup("norm", spec.final_norm.kind)
-        self.final_norm = final_cls(spec.final_norm, spec.hidden_size,
-                                    {"weight": params["final_norm.weight"]}, self.dtype,
-                                    self.device)
+        self.final_norm = final_cls(
+            spec.final_norm, spec.hidden_size,
+            {name: params[f"final_norm.{name}"]
+             for name in final_cls.parameters(spec.final_norm, spec.hidden_size)
+             if f"final_norm.{name}" in params}, self.dtype, self.device)
         if "head.weight" in params and params["head.weight"] is not params["embed.weight"]:
             self.head = Linear(params["head.weight"], self.dtype, self.device,
                                bias=params.get("head.bias"))
@@ -184,6 +186,9 @@ class DecoderModel:
         model is made, where they are not built yet, instead of one after the other at their
         first use."""
         names = ["rowwise", *Linear.kernel_libraries(dtype)]        # embedding, norms, head
+        ask = getattr(lookup("norm", spec.final_norm.kind), "kernel_libraries", None)
+        if ask is not None:
+            names.extend(ask(spec.final_norm, dtype))
         for layer in spec.layers:
             ask = getattr(lookup("block", layer.block), "kernel_libraries", None)
             if ask is not None:

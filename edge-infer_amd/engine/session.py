@@ -172,7 +172,8 @@ class Session:
     def free_tokens(self) -> int:
         if not self.cache.kv_pools:
             return self.cache.n_pages * PAGE_TOKENS
-        return min(pool.n_free for pool in self.cache.kv_pools) * PAGE_TOKENS
+        return min(pool.n_free * pages.stride for pool, pages in
+                   zip(self.cache.kv_pools, self.cache.kv_pages)) * PAGE_TOKENS
 
     # -- generation ----------------------------------------------------------
     def generate_batch(self, prompts, *, max_length=None, max_new_tokens=None, temperature=1.0,

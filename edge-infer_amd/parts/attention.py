@@ -28,9 +28,20 @@ frequencies that may be rescaled, any rotated width, values of their own width),
 the step's source layer computed for the same token, kept in float32 for the step) and
 `output_gate` (the concatenated heads times sigmoid(W_g x), the gate's rows fused into the
 q/k/v product) go through `lib.head_store`, the store kernel for rows that go on after v.
+So do a rotation of neighbouring pairs (position kind "rope_pairs": a query and a key give
+the same score when both are permuted alike, so the rows of the q and k projections are
+reordered when the part is built, evens then odds within a head's rotated part, and the
+rotation of halves does the rest), `query_temperature` (queries grow with the position),
+`output_gate = "head"` (one gate a head, applied by the attention kernel), `shared_kv` (a part
+without key and value projections, whose runs read what another run cached) and `pool`
+(besides its window a query sees one key and value, the means, for every block of `pool`
+positions that lies wholly before the window: the part keeps them in a second paged cache of
+its own, one entry a block, which `lib.pool_store` fills from the cached tokens as blocks
+become complete, and the generic kernel walks after the window).
 """
 from __future__ import annotations
 
+import dataclasses
 import functools
 import os
 
@@ -86,18 +97,17 @@ class Attention:
 
     @classmethod
     def parameters(cls, spec, hidden):
-        params = {
-            "q_proj.weight": ParamSpec((spec.q_width, hidden)),
-            "k_proj.weight": ParamSpec((spec.kv_width, hidden)),
-            "v_proj.weight": ParamSpec((spec.v_width, hidden)),
-            "o_proj.weight": ParamSpec((hidden, spec.out_width)),
-        }
+        params = {"q_proj.weight": ParamSpec((spec.q_width, hidden)),
+                  "o_proj.weight": ParamSpec((hidden, spec.out_width))}
+        if not spec.shared_kv:
+            params["k_proj.weight"] = ParamSpec((spec.kv_width, hidden))
+            params["v_proj.weight"] = ParamSpec((spec.v_width, hidden))
         if spec.o_bias is not False:
             params["o_proj.bias"] = ParamSpec((hidden,), optional=spec.o_bias is not True)
         if spec.talking_heads:
             params["talk"] = ParamSpec((spec.n_heads, spec.n_heads), init="near_identity",
                                        scale=0.2)
-        if spec.qkv_bias is not False:
+        if spec.qkv_bias is not False and not spec.shared_kv:
             required = spec.qkv_bias is True
             params["q_proj.bias"] = ParamSpec((spec.q_width,), optional=not required)
             params["k_proj.bias"] = ParamSpec((spec.kv_width,), optional=not required)
@@ -115,14 +125,34 @@ class Attention:
             params["value_mix"] = ParamSpec((), init="uniform", low=0.1, high=0.6,
                                             optional=spec.value_mix != "mix")
         if spec.output_gate:
-            params["gate_proj.weight"] = ParamSpec((spec.out_width, hidden))
+            rows = spec.n_heads if spec.output_gate == "head" else spec.out_width
+            params["gate_proj.weight"] = ParamSpec((rows, hidden))
         return params
 
     @classmethod
     def cache_request(cls, spec):
-        return KVRequest(n_kv_heads=spec.n_kv_heads, head_dim=spec.head_dim, window=spec.window,
+        # positions the cache keeps behind the newest one: the window's, and the block's that
+        # the newest position may complete; more where other runs read with a wider mask
+        keep = spec.window
+        if keep is not None and spec.pool is not None:
+            keep = max(keep, spec.pool)
+        if spec.cache_span is not None:
+            keep = None if spec.cache_span == 0 or keep is None else max(keep, spec.cache_span)
+        return KVRequest(n_kv_heads=spec.n_kv_heads, head_dim=spec.head_dim, window=keep,
                          value_dim=None if spec.v_dim == spec.head_dim else spec.v_dim,
                          chunk=spec.chunk)
+
+    POOL = "pool"      # the name of the pooled cache under the run's own cache id
+
+    @classmethod
+    def own_cache_request(cls, spec):
+        """What a run keeps for itself even when it reads another run's keys and values: the
+        pooled blocks, which depend on its own block size."""
+        if spec.pool is None:
+            return None
+        return {cls.POOL: KVRequest(n_kv_heads=spec.n_kv_heads, head_dim=spec.head_dim,
+                                    value_dim=None if spec.v_dim == spec.head_dim else spec.v_dim,
+                                    stride=spec.pool)}
 
     @classmethod
     def kernel_libraries(cls, spec, dtype):
@@ -130,7 +160,7 @@ class Attention:
         step."""
         group = spec.n_heads // max(1, spec.n_kv_heads)
         fast = (dtype == torch.bfloat16 and spec.v_dim == spec.head_dim and MATRIX_CORE_ATTENTION
-                and not spec.talking_heads
+                and not spec.talking_heads and spec.pool is None and spec.output_gate != "head"
                 and lib.attention_decode_mfma_supported(spec.head_dim, group))
         kernels = "attention_mfma" if fast else "attention_generic"
         if cls.wide_keys(spec, dtype):
@@ -149,8 +179,9 @@ class Attention:
     @classmethod
     def general_store(cls, spec) -> bool:
         """Whether the part norms, rotates and stores through `lib.head_store`."""
-        return (spec.position.kind == "rope_half" or spec.value_mix in ("source", "mix")
-                or spec.output_gate)
+        return (spec.position.kind in ("rope_half", "rope_pairs")
+                or spec.value_mix in ("source", "mix") or bool(spec.output_gate)
+                or spec.query_temperature is not None or spec.shared_kv or spec.pool is not None)
 
     @classmethod
     def check(cls, spec):
@@ -162,9 +193,9 @@ class Attention:
         if spec.value_mix not in (None, "off", "source", "mix"):
             raise ValueError(f"attention: unknown value_mix '{spec.value_mix}'")
         if cls.general_store(spec):
-            if spec.position.kind not in ("rope_half", "none"):
+            if spec.position.kind not in ("rope_half", "rope_pairs", "none"):
                 raise ValueError("attention: value mixing and the output gate are implemented "
-                                 "with position kinds 'rope_half' and 'none'")
+                                 "with position kinds 'rope_half', 'rope_pairs' and 'none'")
             if spec.qk_norm and spec.qk_norm_scope != "head":
                 raise ValueError("attention: this store norms per head only")
             if spec.talking_heads or spec.qkv_bias:
@@ -197,6 +228,19 @@ class Attention:
             raise ValueError("attention: talking heads with a distance term are not implemented")
         if spec.window is not None and spec.window < 1:
             raise ValueError("attention: a window must be at least 1")
+        if spec.output_gate not in (False, True, "head"):
+            raise ValueError(f"attention: unknown output_gate {spec.output_gate!r}")
+        if spec.pool is not None:
+            if spec.pool < 1 or spec.window is None:
+                raise ValueError("attention: pooled blocks hold at least one position and need "
+                                 "a window")
+            if spec.chunk is not None or spec.talking_heads or spec.distance_slope_range is not None:
+                raise ValueError("attention: pooled blocks with chunks, mixed scores or a "
+                                 "distance term are not implemented")
+        if spec.query_temperature is not None and spec.query_temperature[1] < 1:
+            raise ValueError("attention: the query temperature's step must be at least 1")
+        if spec.shared_kv and spec.value_mix in ("source", "mix"):
+            raise ValueError("attention: a part without values of its own mixes none")
         if spec.chunk is not None and spec.chunk < 1:
             raise ValueError("attention: a chunk must hold at least one position")
 
@@ -205,10 +249,20 @@ class Attention:
         self.spec = spec
         self.hidden = hidden
         self.dtype = dtype
-        fused = torch.cat([params["q_proj.weight"], params["k_proj.weight"],
-                           params["v_proj.weight"]]
+        q_weight = params["q_proj.weight"]
+        k_weight = None if spec.shared_kv else params["k_proj.weight"]
+        position_spec = spec.position
+        if spec.position.kind == "rope_pairs":
+            # neighbouring pairs (2i, 2i + 1) become the pairs (i, i + R/2) of permuted rows
+            order = self._pairs_to_halves(spec.head_dim, spec.position.dim)
+            q_weight = self._permute_heads(q_weight, spec.n_heads, order)
+            if k_weight is not None:
+                k_weight = self._permute_heads(k_weight, spec.n_kv_heads, order)
+            position_spec = dataclasses.replace(spec.position, kind="rope_half", scaling=None)
+        fused = torch.cat([q_weight]
+                          + ([] if spec.shared_kv else [k_weight, params["v_proj.weight"]])
                           + ([params["gate_proj.weight"]] if spec.output_gate else []), dim=0)
-        names = ("q_proj", "k_proj", "v_proj")
+        names = ("q_proj",) if spec.shared_kv else ("q_proj", "k_proj", "v_proj")
         fused_bias = None
         if any(f"{name}.bias" in params for name in names):   # absent ones count as zero
             fused_bias = torch.cat([
@@ -221,7 +275,7 @@ class Attention:
         if spec.qk_norm:
             self.q_norm = params["q_norm.weight"].to(device=device, dtype=torch.float32).contiguous()
             self.k_norm = params["k_norm.weight"].to(device=device, dtype=torch.float32).contiguous()
-        self.position = positions(spec.position)   # shared table object
+        self.position = positions(position_spec)   # shared table object
         self.group = spec.n_heads // spec.n_kv_heads
         self.scale = spec.scale if spec.scale is not None else spec.head_dim ** -0.5
         # without a rotation and without per-head norms, one kernel norms (or not) and stores
@@ -231,7 +285,11 @@ class Attention:
         self.value_lambda = None
         if spec.value_mix == "mix":
             self.value_lambda = params["value_mix"].to(device=device, dtype=torch.float32).reshape(1).contiguous()
-        self.gate_column = spec.q_width + spec.kv_width + spec.v_width    # where the gate's columns begin
+        # kv heads whose keys and values the rows of this part's projection hold
+        self.own_kv_heads = 0 if spec.shared_kv else spec.n_kv_heads
+        # where the gate's columns begin
+        self.gate_column = spec.q_width + (0 if spec.shared_kv else spec.kv_width + spec.v_width)
+        self.head_gate = spec.output_gate == "head"
         self.slopes = self.sinks = None
         if spec.distance_slope_range is not None:
             exponent = -float(spec.distance_slope_range) * torch.arange(
@@ -248,6 +306,7 @@ class Attention:
         # as the keys; every other case runs the generic kernel
         self.matrix_cores = (dtype == torch.bfloat16 and spec.v_dim == spec.head_dim and
                             MATRIX_CORE_ATTENTION and self.talk is None and
+                            spec.pool is None and not self.head_gate and
                             lib.attention_decode_mfma_supported(spec.head_dim, self.group))
         # chunk, slopes, sink: what the kernels take beyond a window
         self.wide = self.wide_keys(spec, dtype)
@@ -255,6 +314,20 @@ class Attention:
         self.has_extras = spec.chunk is not None or self.slopes is not None or self.sinks is not None
         self.compute_units = lib.compute_units(device)     # the chip's size, for launch plans
         self._decode_launches = {}     # (sequences, pages of context) -> decode_launch's answer
+
+    @staticmethod
+    def _pairs_to_halves(head_dim: int, rotated: int):
+        """Order of a head's rows after which the rotation of the pairs (i, i + R/2) turns what
+        the rotation of the neighbours (2i, 2i + 1) turned: the even rows of the rotated part,
+        then its odd rows, then the rest."""
+        return list(range(0, rotated, 2)) + list(range(1, rotated, 2)) + list(range(rotated, head_dim))
+
+    @staticmethod
+    def _permute_heads(weight, heads: int, order):
+        head_dim = len(order)
+        index = torch.tensor([head * head_dim + row for head in range(heads) for row in order],
+                             dtype=torch.long, device=weight.device)
+        return weight.index_select(0, index)
 
     # the number of positions of one sequence that a prefill work item covers
     def positions_per_item(self, key_ways: int = 1):
@@ -394,6 +467,7 @@ class Attention:
         # (the kernel that norms and stores the whole projection adds its bias as well)
         qkv, bias = (self.qkv.forward(ctx, x, "attn.qkv", bias_later=True) if self.whole_store
                      else (self.qkv.forward(ctx, x, "attn.qkv"), None))
+        gate, pooled = None, {}
         if self.general:
             q = ctx.buffer("attn.q", (n, spec.q_width))
             v_first, v_mode = None, 0
@@ -408,12 +482,25 @@ class Attention:
                     raise ValueError("attention: a layer mixes values in, but no earlier layer of "
                                      "the step has kept values of that width")
                 v_mode = 2
+            if self.head_gate:
+                gate = ctx.buffer("attn.gate", (n, spec.n_heads), torch.float32)
+            if entry.writes_cache and spec.shared_kv:
+                raise ValueError("attention: a part without key and value projections cannot "
+                                 "write a cache entry")
             lib.head_store(qkv, self.q_norm, self.k_norm, spec.qk_norm_eps,
                            getattr(self.position, "frequencies", None), meta.row_pos,
                            meta.row_seq, page_table, q, k_pages, v_pages, spec.n_heads,
-                           spec.n_kv_heads, spec.head_dim, spec.v_dim,
+                           self.own_kv_heads, spec.head_dim, spec.v_dim,
                            write_cache=entry.writes_cache, v_first=v_first, v_mode=v_mode,
-                           v_lambda=self.value_lambda)
+                           v_lambda=self.value_lambda, query_temperature=spec.query_temperature,
+                           gate_out=gate, gate_column=self.gate_column)
+            if spec.pool is not None:
+                # the blocks that this step's rows complete, from the keys as the cache holds them
+                pool_group, pool_k, pool_v = ctx.cache.kv((entry.own_id, self.POOL))
+                pool_table = meta.page_table(pool_group)
+                lib.pool_store(k_pages, v_pages, meta.row_pos, meta.row_seq, page_table,
+                               pool_table, pool_k, pool_v, n, spec.pool)
+                pooled = dict(pool=spec.pool, pool_k=pool_k, pool_v=pool_v, pool_table=pool_table)
         elif (ctx.decode and self.matrix_cores and FUSED_DECODE and qkv.dim() == 3
                 and qkv.dtype == torch.float32 and not self.whole_store and not self.has_extras):
             # the decode kernel norms, rotates and stores for its rows itself: one launch less
@@ -439,7 +526,7 @@ class Attention:
             q = mixed
         out = ctx.buffer("attn.out", (n, spec.out_width))
         more = dict(value_dim=spec.v_dim, key_heads=1 if self.talk is None else spec.n_kv_heads,
-                    **self.extras)
+                    gate=gate, **pooled, **self.extras)
         part_o = part_ml = None
         if ctx.decode:
             splits, waves, heads = self._decode_launch_for(ctx.n_seqs, ctx.context_bound)
@@ -497,9 +584,9 @@ class Attention:
                               meta.row_pos, meta.row_seq, page_table, out, spec.n_heads,
                               spec.n_kv_heads, spec.head_dim, window=spec.window,
                               scale=self.scale, **more)
-        if spec.output_gate:
+        if spec.output_gate and not self.head_gate:
             lib.gate_rows(qkv, self.gate_column, out)
-        ctx.release(qkv, None if isinstance(q, lib.DecodeProjection) else q, part_o, part_ml)
+        ctx.release(qkv, None if isinstance(q, lib.DecodeProjection) else q, part_o, part_ml, gate)
         delta = self.o.forward(ctx, out, "attn.o", bias_later=bias_later)
         ctx.release(out)
         return delta

@@ -27,12 +27,20 @@ class KVRequest:
     """Keys and values for every position (or the last `window`) of a sequence: pages
     [kv_heads, 64, head_dim] of keys and [kv_heads, 64, value_dim] of values (`value_dim`
     None: as wide as the keys).  `chunk`: a query sees only keys of its own block of that many
-    positions, so pages that lie wholly before the block of the next position are given back."""
+    positions, so pages that lie wholly before the block of the next position are given back.
+    `stride` s > 1: the entry holds one key and value for every complete block of s positions
+    (what a mixer derives from the tokens of the block), so a sequence of n tokens holds
+    n // s of them, in pages of 64 like any other.
+
+    A mixer (or a block arrangement) that needs several things asks for a dictionary
+    {name: request}; the thing called `name` of cache entry `id` is then found under the id
+    `(id, name)` (the name "" stands for `id` itself), and a dictionary may hold dictionaries."""
     n_kv_heads: int
     head_dim: int
     window: Optional[int] = None
     value_dim: Optional[int] = None
     chunk: Optional[int] = None
+    stride: int = 1
 
 
 @dataclass(frozen=True)

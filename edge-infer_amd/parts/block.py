@@ -5,6 +5,7 @@ import torch
 
 from ..csrc import lib
 from ..weights.loader import ParamSpec
+from .base import StateRequest
 from .registry import lookup
 
 
@@ -205,8 +206,16 @@ class SandwichBlock:
     and a norm after every sublayer, and a multiplier s (`residual_scale`) on what is added.  A
     layer may have no feed-forward (then it has no second pair of norms either).
 
-    The multiplier is folded into the float32 weights of the norms on the outputs when the
-    block is built.  The norm on the mixer's output, the addition and the feed-forward's input
+    Options of the layer spec: `layer_scale`: what a sublayer adds is also multiplied, element
+    by element, by a learned vector (`scale1` for the mixer, `scale2` for the feed-forward);
+    `input_conv` T > 0: what a sublayer reads, h = norm(x), becomes h + conv(h), a causal
+    convolution over time on every channel with a learned filter [width, T] (`conv1.weight`,
+    `conv2.weight`); the last T - 1 inputs of both sublayers are state of the sequence, which
+    the block keeps under the run's own cache id (`own_cache_request`), so a prompt may come
+    whole, in portions or token by token.
+
+    The multipliers are folded into the float32 weights (and biases) of the norms on the
+    outputs when the block is built.  The norm on the mixer's output, the addition and the feed-forward's input
     norm are one kernel; everything is added when the block returns, so it returns no pending
     delta and follows only blocks that do the same."""
 
@@ -243,7 +252,37 @@ class SandwichBlock:
                 for name, param in norm_cls.parameters(layer_spec.norm, hidden).items():
                     params[f"{prefix}.{name}"] = ParamSpec(param.shape, init=param.init,
                                                            optional=True)
+        both = layer_spec.feed_forward is not None
+        if getattr(layer_spec, "layer_scale", False):
+            params["scale1"] = ParamSpec((hidden,), init="uniform", low=0.5, high=1.5)
+            params["scale2"] = ParamSpec((hidden,), init="uniform", low=0.5, high=1.5,
+                                         optional=not both)
+        taps = getattr(layer_spec, "input_conv", 0)
+        if taps:
+            params["conv1.weight"] = ParamSpec((hidden, taps), scale=0.3)
+            params["conv2.weight"] = ParamSpec((hidden, taps), scale=0.3, optional=not both)
         return params
+
+    CONV_STATE = "input_conv"      # the name of the block's state under the run's own cache id
+
+    @classmethod
+    def own_cache_request(cls, layer_spec):
+        """What a run of this layer keeps for itself, whichever cache entry its mixer uses:
+        the last taps - 1 inputs of both convolutions, [2, taps - 1, width] floats a sequence
+        (two versions: a step reads one and writes the other)."""
+        taps = getattr(layer_spec, "input_conv", 0)
+        if taps <= 1:
+            return None
+        return {cls.CONV_STATE: StateRequest(shape=(2 * (taps - 1) * cls._width_of(layer_spec),),
+                                             two_versions=True)}
+
+    @staticmethod
+    def _width_of(layer_spec):
+        width = getattr(layer_spec, "width", None)
+        if width is None:
+            raise ValueError("sandwich: a layer with an input convolution must name the model's "
+                             "width (LayerSpec.width)")
+        return int(width)
 
     @classmethod
     def mixer_spec(cls, layer_spec):
@@ -252,6 +291,8 @@ class SandwichBlock:
     @classmethod
     def kernel_libraries(cls, layer_spec, dtype):
         names = ["rowwise"]
+        if getattr(layer_spec, "input_conv", 0):
+            names.append("input_conv")
         for _, owner, spec in cls._owners(layer_spec):
             ask = getattr(owner, "kernel_libraries", None)
             if ask is not None:
@@ -266,32 +307,66 @@ class SandwichBlock:
         if not hasattr(norm_cls, "norm_add"):
             raise ValueError(f"norm kind '{layer_spec.norm.kind}' cannot sit on a sublayer's output")
         scale = float(layer_spec.residual_scale)
+        layer_scale = getattr(layer_spec, "layer_scale", False)
 
-        def after(prefix):
-            """The norm on a sublayer's output, with the multiplier in its weight."""
+        def after(prefix, vector_name):
+            """The norm on a sublayer's output, with the multipliers in its weight."""
             norm = norm_cls(layer_spec.norm, hidden, sub(prefix), dtype, device)
-            if scale != 1.0:
-                norm.weight = (norm.weight * scale).contiguous()
+            factor = None if scale == 1.0 else scale
+            if layer_scale:
+                vector = params[vector_name].to(device=device, dtype=torch.float32)
+                factor = vector if factor is None else vector * factor
+            if factor is not None:
+                if hasattr(norm, "scale_by"):
+                    norm.scale_by(factor)
+                else:
+                    norm.weight = (norm.weight * factor).contiguous()
             return norm
         self.norm1 = norm_cls(layer_spec.norm, hidden, sub("norm1"), dtype, device)
         self.mixer = lookup("mixer", layer_spec.mixer.kind)(
             layer_spec.mixer, hidden, sub("mixer"), dtype, device, positions=positions)
-        self.norm1b = after("norm1b")
+        self.norm1b = after("norm1b", "scale1")
         self.norm2 = self.ffn = self.norm2b = None
         if layer_spec.feed_forward is not None:
             self.norm2 = norm_cls(layer_spec.norm, hidden, sub("norm2"), dtype, device)
             self.ffn = lookup("feed_forward", layer_spec.feed_forward.kind)(
                 layer_spec.feed_forward, hidden, sub("ffn"), dtype, device)
-            self.norm2b = after("norm2b")
-        # the fused kernel takes two plain RMS norms of one eps
+            self.norm2b = after("norm2b", "scale2")
+        # one kernel for the norm on the mixer's output, the addition and the next norm: two
+        # plain RMS norms of one eps, or norms that bring such a kernel themselves
         self.fused = all(hasattr(norm, "weight") and hasattr(norm, "eps")
+                         and not getattr(norm, "centred", False)
                          for norm in (self.norm1b, self.norm2) if norm is not None)
+        self.fused_own = (self.norm2 is not None and hasattr(self.norm1b, "norm_add_then")
+                          and type(self.norm1b) is type(self.norm2))
+        self.taps = int(getattr(layer_spec, "input_conv", 0))
+        self.conv1 = self.conv2 = None
+        if self.taps:
+            self.conv1 = params["conv1.weight"].to(device=device, dtype=torch.float32).contiguous()
+            if self.ffn is not None:
+                self.conv2 = params["conv2.weight"].to(device=device, dtype=torch.float32).contiguous()
+
+    def _convolved(self, ctx, h, entry, part):
+        """h + conv(h) for sublayer `part` (0: the mixer, 1: the feed-forward)."""
+        meta = ctx.meta
+        out = ctx.buffer("block.hc", tuple(h.shape))
+        state = seq_in = seq_out = None
+        if self.taps > 1:
+            state = ctx.cache.state((entry.own_id, self.CONV_STATE))
+            seq_in, seq_out = meta.seq_state_in, meta.seq_state_out
+        lib.input_conv(h, self.conv1 if part == 0 else self.conv2, state, part, 2, meta.row_pos,
+                       meta.row_seq, seq_in, seq_out, meta.seq_start, meta.seq_count,
+                       meta.seq_row0, out)
+        ctx.release(h)
+        return out
 
     def forward(self, ctx, residual, pending, entry):
         if pending is not None:
             raise ValueError("sandwich: a delta of the block before is still pending; this "
                              "arrangement follows only blocks that add everything themselves")
         h = self.norm1.add_norm(ctx, residual, None, "block.h", write_residual=False)
+        if self.taps:
+            h = self._convolved(ctx, h, entry, 0)
         # a sublayer that can leave its last product's bias to the norm kernel behind it does
         a, a_bias = (self.mixer.forward(ctx, h, entry, bias_later=True)
                      if getattr(self.mixer, "bias_later", False)
@@ -305,10 +380,14 @@ class SandwichBlock:
             h2 = ctx.buffer("block.h", tuple(residual.shape))
             lib.norm_add_norm(residual, a, self.norm1b.weight, self.norm2.weight, self.norm2.eps, h2,
                               bias=a_bias)
+        elif self.fused_own:
+            h2 = self.norm1b.norm_add_then(ctx, residual, a, self.norm2, "block.h", bias=a_bias)
         else:
             self.norm1b.norm_add(ctx, residual, a, bias=a_bias)
             h2 = self.norm2.add_norm(ctx, residual, None, "block.h", write_residual=False)
         ctx.release(a)
+        if self.taps:
+            h2 = self._convolved(ctx, h2, entry, 1)
         f, f_bias = (self.ffn.forward(ctx, h2, bias_later=True)
                      if getattr(self.ffn, "bias_later", False)
                      else (self.ffn.forward(ctx, h2), None))
