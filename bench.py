@@ -2,7 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L]
                     [--shape 8b|0.6b|32b] [--only decode|prefill|generate] [--prompt P]
-                    [--with-32b] [--peaks] [--design tirurax|zadenex|vafepel [--design-shape 1k|2k|4k]]
+                    [--with-32b] [--peaks] [--design tirurax|zadenex|vafepel|gopuzen [--design-shape 1k|2k|4k]]
 
 Prints one JSON line.  `value` is decoded tokens per second at the given batch after
 512-token prompts (one step = one decode step of the whole batch: the model, greedy
@@ -30,7 +30,12 @@ heads, gated feed-forward, one pass of a loop over the last six layers) beside t
 model of the same width, layers, heads and parameter count.  `--design vafepel` does the same
 for a Vafepel model (state-space and window-attention layers in turn, the feed-forwards in
 turn dense and routed over 8 experts) beside the Tirurax model of the same width, layers,
-heads and parameters at work for a token.
+heads and parameters at work for a token.  `--design gopuzen` does the same for a Gopuzen model
+(layers of softmax attention beside linear attention and layers of window attention with pooled
+blocks in turn, every second of the latter reading the keys and values of the one before it;
+layer norms on both sides of every sublayer, input convolutions, the feed-forwards in turn
+dense and routed over 8 experts and 2 identity experts) beside the Vafepel model of the same
+width, layers, heads and parameters at work for a token.
 Synthetic token ids, seeded random weights N(0, 0.02).  Peaks are the MI355X's published
 ones: HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s; `measured_peaks` (and `--peaks` alone) say what
 a plain read kernel and a loop of matrix-core products reach on the GPU at hand, and the
@@ -449,6 +454,49 @@ def vafepel_configs(shape):
     return new, old
 
 
+def gopuzen_configs(shape):
+    """(Gopuzen configuration, Vafepel configuration) of equal width, layers, heads, head size
+    and feed-forward parameters at work for a token: a layer of softmax attention (no
+    rotation, queries that grow with the position) beside linear attention with a decay per
+    head stands where a state-space layer stands, window attention with a rotation of half the
+    head, pooled blocks of 64 tokens before the window and a gate per head where window
+    attention stands (every second such layer reads the keys and values of the one before
+    it); the feed-forwards are in turn the dense gated one and 8 experts of half its width
+    (and 2 identity experts) of which a token takes 2."""
+    from edge_infer_amd.config import GopuzenConfig
+    layers, width, d_heads, d_kv, a_heads, a_kv, dim, chunk, vocab = DESIGN_SHAPES[shape]
+    ff = 4 * width
+    gated = (2 * ff // 3 + 255) // 256 * 256
+    dense = {"kind": "dense", "ff": gated}
+    routed = {"kind": "moe", "expert": {"ff": gated // 2},
+              "router": {"experts": 8, "top": 2, "identity": 2}}
+    decay = [1.0 - 2.0 ** (-5.0 - 4.0 * h / max(1, d_heads - 1)) for h in range(d_heads)]
+    parallel = {"type": "parallel",
+                "mixer": {"left": {"heads": a_heads, "kv_heads": a_kv, "dim": dim, "vdim": dim,
+                                   "scale": dim ** -0.5, "q_temp": {"coef": 0.1, "every": 1024}},
+                          "right": {"heads": d_heads, "dim": dim, "vdim": dim, "decay": decay}}}
+    window = {"heads": a_heads, "kv_heads": a_kv, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
+              "mask": {"size": chunk, "pool": 64}, "rot": {"base": 500000.0, "dims": dim // 2}}
+    order, last_window = [], None
+    for i in range(layers):
+        mlp = dense if i % 4 < 2 else routed
+        if i % 2 == 0:
+            order.append(dict(parallel, mlp=mlp))
+            continue
+        mixer = dict(window)
+        if last_window is not None:
+            mixer["kv_from"] = last_window
+            last_window = None
+        else:
+            last_window = i
+        order.append({"type": "attention", "mixer": mixer, "mlp": mlp})
+    new = GopuzenConfig.from_dict({"architecture": "Gopuzen", "vocab": vocab, "width": width,
+                                   "norm": {"eps": 1e-6}, "embedding": {"scale": 1.0},
+                                   "canon": {"taps": 4}, "layers": order})
+    old, _ = vafepel_configs(shape)
+    return new, old
+
+
 def measure_prompts(model, vocab, batch, tokens, repeats=3):
     """Best ms of one step over `batch` prompts of `tokens` tokens that start together."""
     import types
@@ -484,6 +532,9 @@ def design_comparison(args):
     elif args.design == "vafepel":
         new, old = vafepel_configs(args.design_shape)
         which = {"vafepel": new, "tirurax": old}
+    elif args.design == "gopuzen":
+        new, old = gopuzen_configs(args.design_shape)
+        which = {"gopuzen": new, "vafepel": old}
     else:
         new, old = design_configs(args.design_shape)
         which = {"tirurax": new, "qwen3": old}
@@ -543,12 +594,12 @@ def main():
                         help="leave the 32B shape (decode at batch 1 and 16, prefill) out of `points`")
     parser.add_argument("--peaks", action="store_true",
                         help="measure the read and matrix-core yardsticks only")
-    parser.add_argument("--design", choices=["tirurax", "zadenex", "vafepel"], default=None,
+    parser.add_argument("--design", choices=["tirurax", "zadenex", "vafepel", "gopuzen"], default=None,
                         help="measure this design beside the closest other model of equal size "
                              "(tirurax beside qwen3, zadenex beside tirurax) instead of the "
                              "default workload")
     parser.add_argument("--design-shape", choices=sorted(DESIGN_SHAPES), default="2k")
-    parser.add_argument("--design-only", choices=["vafepel", "zadenex", "tirurax", "qwen3"], default=None,
+    parser.add_argument("--design-only", choices=["gopuzen", "vafepel", "zadenex", "tirurax", "qwen3"], default=None,
                         help="with --design: one of the two models only (for profiling)")
     args = parser.parse_args()
     if args.gpus != 1:

@@ -12,8 +12,8 @@ their caches.  Beyond the reference, a session can serve a batch of prompts
 (`new_session(max_batch=8)`, `session.generate_batch`) and exposes the step function
 (`session.step`).  Model types: "qwen3_bf16" (the reference's name) and
 "qwen3_fp32" for the true 32-bit path; "tirurax_bf16" / "tirurax_fp32" and "zadenex_bf16" /
-"zadenex_fp32" and "vafepel_bf16" / "vafepel_fp32" likewise for Tirurax, Zadenex and Vafepel
-folders.
+"zadenex_fp32", "vafepel_bf16" / "vafepel_fp32" and "gopuzen_bf16" / "gopuzen_fp32" likewise for
+Tirurax, Zadenex, Vafepel and Gopuzen folders.
 
 The reference's procedural wrappers over one implicit session are here too
 (model_bridge.cpp:159-215,274-283): `init_model`, `generate_text_stream`,
@@ -38,7 +38,8 @@ from .weights import read_tensors
 MODEL_TYPES = {"qwen3_bf16": "bfloat16", "qwen3_fp32": "float32",
                "tirurax_bf16": "bfloat16", "tirurax_fp32": "float32",
                "zadenex_bf16": "bfloat16", "zadenex_fp32": "float32",
-               "vafepel_bf16": "bfloat16", "vafepel_fp32": "float32"}
+               "vafepel_bf16": "bfloat16", "vafepel_fp32": "float32",
+               "gopuzen_bf16": "bfloat16", "gopuzen_fp32": "float32"}
 DEFAULT_CAPACITY = 4096   # bindings/python/model_bridge.cpp:135-141: min(4096, model limit)
 
 

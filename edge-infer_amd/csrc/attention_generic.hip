@@ -377,7 +377,7 @@ extern "C" int ei_attention(const void* q, const void* k_pages, const void* v_pa
 // positions b P .. b P + P - 1 of a sequence, for every kv head.  A wave a (row, kv head): the
 // row at position p with (p + 1) % P == 0 completes block p / P, whose keys all lie in the
 // token cache by then (this step's store has run), and writes the block's entry; every other
-// row has nothing to do.  Sums are float32, in the order of the positions.
+// row has nothing to do.  Sums are float32, in the order of the positions, divided by P.
 namespace {
 
 template <typename T>
@@ -387,35 +387,45 @@ __global__ void pool_store_kernel(const T* __restrict__ k_pages, const T* __rest
                                   const int32_t* __restrict__ page_table,
                                   const int32_t* __restrict__ pool_table, int table_width,
                                   T* __restrict__ pool_k, T* __restrict__ pool_v, int N, int nkv,
-                                  int D, int DV, int P) {
+                                  int D, int DV, int P, int pieces) {
+  // a wave a (row, kv head, piece of 64 elements of [key | value]); eight positions' loads
+  // are issued before the first is added
   const int wave = (blockIdx.x * blockDim.x + threadIdx.x) / EI_WAVE;
   const int lane = threadIdx.x % EI_WAVE;
-  if (wave >= N * nkv) return;
-  const int row = wave / nkv, g = wave % nkv;
+  if (wave >= N * nkv * pieces) return;
+  const int piece = wave % pieces, g = wave / pieces % nkv, row = wave / pieces / nkv;
   const int seq = row_seq[row];
   if (seq < 0) return;
   const int pos = row_pos[row];
   if ((pos + 1) % P != 0) return;
+  const int e = piece * EI_WAVE + lane;
+  if (e >= D + DV) return;
   const int block = pos / P;
   const int32_t* pages = page_table + static_cast<size_t>(seq) * table_width;
   const int dst_page = pool_table[static_cast<size_t>(seq) * table_width + block / EI_PAGE];
   if (dst_page < 0) return;
   const size_t dst = (static_cast<size_t>(dst_page) * nkv + g) * EI_PAGE + block % EI_PAGE;
-  const float share = 1.0f / static_cast<float>(P);
-  for (int e = lane; e < D + DV; e += EI_WAVE) {
-    const bool key = e < D;
-    const int width = key ? D : DV, at = key ? e : e - D;
-    const T* source = key ? k_pages : v_pages;
-    float sum = 0.f;
-    for (int j = 0; j < P; ++j) {
-      const int p = block * P + j;
-      const int phys = pages[p / EI_PAGE];
-      if (phys >= 0)
-        sum += ei::to_f32<T>(source[((static_cast<size_t>(phys) * nkv + g) * EI_PAGE + p % EI_PAGE) *
-                                    width + at]);
+  const bool key = e < D;
+  const int width = key ? D : DV, at = key ? e : e - D;
+  const T* source = key ? k_pages : v_pages;
+  float sum = 0.f;
+  for (int j0 = 0; j0 < P; j0 += 8) {
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      v[u] = 0.f;
+      const int p = block * P + j0 + u;
+      if (j0 + u < P) {
+        const int phys = pages[p / EI_PAGE];
+        if (phys >= 0)
+          v[u] = ei::to_f32<T>(source[((static_cast<size_t>(phys) * nkv + g) * EI_PAGE + p % EI_PAGE) *
+                                      width + at]);
+      }
     }
-    (key ? pool_k : pool_v)[dst * width + at] = ei::from_f32<T>(sum * share);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) sum += v[u];
   }
+  (key ? pool_k : pool_v)[dst * width + at] = ei::from_f32<T>(sum / static_cast<float>(P));
 }
 
 }  // namespace
@@ -431,18 +441,20 @@ extern "C" int ei_pool_store(const void* k_pages, const void* v_pages, int dtype
              "pool_store: null pointer");
   EI_REQUIRE(N > 0 && nkv > 0 && D > 0 && DV > 0 && P >= 1 && table_width > 0,
              "pool_store: sizes must be positive");
-  const size_t waves = static_cast<size_t>(N) * nkv;
+  const int pieces = (D + DV + EI_WAVE - 1) / EI_WAVE;
+  const size_t waves = static_cast<size_t>(N) * nkv * pieces;
+  EI_REQUIRE(waves * EI_WAVE / 256 < 0x7fffffffULL, "pool_store: too many rows for one launch");
   const unsigned blocks = static_cast<unsigned>((waves * EI_WAVE + 255) / 256);
   if (dtype == EI_F32)
     pool_store_kernel<float><<<blocks, 256, 0, stream>>>(
         static_cast<const float*>(k_pages), static_cast<const float*>(v_pages), row_pos, row_seq,
         page_table, pool_table, table_width, static_cast<float*>(pool_k),
-        static_cast<float*>(pool_v), N, nkv, D, DV, P);
+        static_cast<float*>(pool_v), N, nkv, D, DV, P, pieces);
   else if (dtype == EI_BF16)
     pool_store_kernel<bf16_t><<<blocks, 256, 0, stream>>>(
         static_cast<const bf16_t*>(k_pages), static_cast<const bf16_t*>(v_pages), row_pos, row_seq,
         page_table, pool_table, table_width, static_cast<bf16_t*>(pool_k),
-        static_cast<bf16_t*>(pool_v), N, nkv, D, DV, P);
+        static_cast<bf16_t*>(pool_v), N, nkv, D, DV, P, pieces);
   else
     EI_REQUIRE(false, "pool_store: unknown dtype");
   EI_LAUNCH_CHECK();

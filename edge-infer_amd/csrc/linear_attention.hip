@@ -15,8 +15,7 @@
 namespace {
 
 constexpr int kTile = 16;      // tokens whose operands lie in LDS at a time
-constexpr int kCols = 64;      // columns of S a block owns
-constexpr int kGroups = 4;     // waves of a block: each owns a quarter of the rows of S
+constexpr int kThreads = 256;
 
 template <typename TI>
 __device__ __forceinline__ float sliced(const TI* p, int nsplit, size_t split_stride) {
@@ -27,24 +26,29 @@ __device__ __forceinline__ float sliced(const TI* p, int nsplit, size_t split_st
 
 __device__ __forceinline__ float silu_f32(float x) { return x / (1.0f + expf(-x)); }
 
-// A block a (sequence, head, 64 columns of S).  Thread (c, g): column c, rows g R .. g R + R - 1
-// (R a multiple of 4, kGroups * R >= DK; rows beyond DK hold zeros).
-template <typename TI, int R>
-__global__ void __launch_bounds__(kCols * kGroups)
+// A block a (sequence, head, COLS columns of S).  Thread (c, g): column c, rows g R .. g R + R - 1
+// (R a multiple of 4; the 256 / COLS groups g hold G R >= DK rows; rows beyond DK hold zeros).
+// A tile of 16 tokens' q, k and v lies in LDS while its tokens are walked; the next tile's
+// values are asked of global memory before the walk and wait in registers.
+template <typename TI, int R, int COLS>
+__global__ void __launch_bounds__(kThreads)
 la_scan_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride, size_t row_stride,
                const float* __restrict__ decay, const float* state_in_table, float* state_out_table,
                const int32_t* __restrict__ seq_in, const int32_t* __restrict__ seq_out,
                const int32_t* __restrict__ seq_count, const int32_t* __restrict__ seq_row0,
                float* __restrict__ o_raw, int H, int DK, int DV) {
-  constexpr int DKP = kGroups * R;
+  constexpr int G = kThreads / COLS;
+  constexpr int DKP = G * R;
+  constexpr int QK_PER = kTile * DKP / kThreads;      // q (and k) values a thread fetches a tile
+  constexpr int V_PER = (kTile * COLS + kThreads - 1) / kThreads;
   __shared__ __attribute__((aligned(16))) float qs[kTile][DKP];
   __shared__ __attribute__((aligned(16))) float ks[kTile][DKP];
-  __shared__ float vs[kTile][kCols];
-  __shared__ float part[kTile][kGroups][kCols];
-  const int seq = blockIdx.x, head = blockIdx.y, col0 = blockIdx.z * kCols;
+  __shared__ float vs[kTile][COLS];
+  __shared__ float part[kTile][G][COLS];
+  const int seq = blockIdx.x, head = blockIdx.y, col0 = blockIdx.z * COLS;
   const int count = seq_count[seq];
   if (count <= 0) return;                       // a padding sequence
-  const int t = threadIdx.x, c = t % kCols, g = t / kCols;
+  const int t = threadIdx.x, c = t % COLS, g = t / COLS;
   const int col = col0 + c;
   const bool col_live = col < DV;
   const size_t state_floats = static_cast<size_t>(H) * DK * DV;
@@ -65,33 +69,50 @@ la_scan_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride, siz
   const size_t v_at = 2 * static_cast<size_t>(H) * DK + static_cast<size_t>(head) * DV + col0;
   const size_t out_width = static_cast<size_t>(H) * DV;
 
+  float q_next[QK_PER], k_next[QK_PER], v_next[V_PER];
+  // the raw projections of the tile that starts at `tile0`, into registers
+  auto fetch = [&](int tile0) {
+    const int nt = min(kTile, count - tile0);
+#pragma unroll
+    for (int u = 0; u < QK_PER; ++u) {
+      const int idx = t + u * kThreads, tt = idx / DKP, row = idx % DKP;
+      q_next[u] = k_next[u] = 0.f;
+      if (tt < nt && row < DK) {
+        const TI* src = proj + static_cast<size_t>(row0 + tile0 + tt) * row_stride;
+        q_next[u] = sliced(src + q_at + row, nsplit, split_stride);
+        k_next[u] = sliced(src + k_at + row, nsplit, split_stride);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < V_PER; ++u) {
+      const int idx = t + u * kThreads, tt = idx / COLS, cc = idx % COLS;
+      v_next[u] = 0.f;
+      if (idx < kTile * COLS && tt < nt && col0 + cc < DV)
+        v_next[u] = sliced(proj + static_cast<size_t>(row0 + tile0 + tt) * row_stride + v_at + cc,
+                           nsplit, split_stride);
+    }
+  };
+  fetch(0);
   for (int tile0 = 0; tile0 < count; tile0 += kTile) {
     const int nt = min(kTile, count - tile0);
-    for (int idx = t; idx < nt * DKP; idx += kCols * kGroups) {
-      const int tt = idx / DKP, row = idx % DKP;
-      float qv = 0.f, kv = 0.f;
-      if (row < DK) {
-        const TI* src = proj + static_cast<size_t>(row0 + tile0 + tt) * row_stride;
-        qv = silu_f32(sliced(src + q_at + row, nsplit, split_stride));
-        kv = silu_f32(sliced(src + k_at + row, nsplit, split_stride));
-      }
-      qs[tt][row] = qv;
-      ks[tt][row] = kv;
+#pragma unroll
+    for (int u = 0; u < QK_PER; ++u) {
+      const int idx = t + u * kThreads;
+      qs[idx / DKP][idx % DKP] = silu_f32(q_next[u]);
+      ks[idx / DKP][idx % DKP] = silu_f32(k_next[u]);
     }
-    for (int idx = t; idx < nt * kCols; idx += kCols * kGroups) {
-      const int tt = idx / kCols, cc = idx % kCols;
-      float vv = 0.f;
-      if (col0 + cc < DV)
-        vv = silu_f32(sliced(proj + static_cast<size_t>(row0 + tile0 + tt) * row_stride + v_at + cc,
-                             nsplit, split_stride));
-      vs[tt][cc] = vv;
+#pragma unroll
+    for (int u = 0; u < V_PER; ++u) {
+      const int idx = t + u * kThreads;
+      if (idx < kTile * COLS) vs[idx / COLS][idx % COLS] = silu_f32(v_next[u]);
     }
     __syncthreads();
+    if (tile0 + kTile < count) fetch(tile0 + kTile);
     for (int tt = 0; tt < nt; ++tt) {
       const float vv = vs[tt][c];
       const float4* kq = reinterpret_cast<const float4*>(&ks[tt][g * R]);
       const float4* qq = reinterpret_cast<const float4*>(&qs[tt][g * R]);
-      float acc = 0.f;
+      float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
 #pragma unroll
       for (int i4 = 0; i4 < R / 4; ++i4) {
         const float4 k4 = kq[i4], q4 = qq[i4];
@@ -99,20 +120,20 @@ la_scan_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride, siz
         S[4 * i4 + 1] = d * S[4 * i4 + 1] + k4.y * vv;
         S[4 * i4 + 2] = d * S[4 * i4 + 2] + k4.z * vv;
         S[4 * i4 + 3] = d * S[4 * i4 + 3] + k4.w * vv;
-        acc += S[4 * i4 + 0] * q4.x;
-        acc += S[4 * i4 + 1] * q4.y;
-        acc += S[4 * i4 + 2] * q4.z;
-        acc += S[4 * i4 + 3] * q4.w;
+        a0 += S[4 * i4 + 0] * q4.x;
+        a1 += S[4 * i4 + 1] * q4.y;
+        a2 += S[4 * i4 + 2] * q4.z;
+        a3 += S[4 * i4 + 3] * q4.w;
       }
-      part[tt][g][c] = acc;
+      part[tt][g][c] = (a0 + a1) + (a2 + a3);
     }
     __syncthreads();
-    for (int idx = t; idx < nt * kCols; idx += kCols * kGroups) {
-      const int tt = idx / kCols, cc = idx % kCols;
+    for (int idx = t; idx < nt * COLS; idx += kThreads) {
+      const int tt = idx / COLS, cc = idx % COLS;
       if (col0 + cc < DV) {
         float o = part[tt][0][cc];
 #pragma unroll
-        for (int gg = 1; gg < kGroups; ++gg) o += part[tt][gg][cc];
+        for (int gg = 1; gg < G; ++gg) o += part[tt][gg][cc];
         o_raw[static_cast<size_t>(row0 + tile0 + tt) * out_width + static_cast<size_t>(head) * DV +
               col0 + cc] = o;
       }
@@ -166,19 +187,28 @@ extern "C" int ei_la_scan(const void* proj, int proj_dtype, int nsplit, long lon
   EI_REQUIRE(n_seqs > 0 && H > 0 && DK >= 1 && DK <= 256 && DV >= 1 && nsplit >= 1,
              "la_scan: key heads of 1 to 256 elements");
   EI_REQUIRE(row_stride >= 2LL * H * DK + 1LL * H * DV, "la_scan: rows narrower than q, k and v");
-  EI_REQUIRE(H <= 65535 && (DV + kCols - 1) / kCols <= 65535, "la_scan: too many heads");
-  const dim3 grid(n_seqs, H, (DV + kCols - 1) / kCols);
+  EI_REQUIRE(H <= 65535 && (DV + 15) / 16 <= 65535, "la_scan: too many heads");
+  // 64 columns a block where that fills the chip; 16 (and a quarter of the rows a thread)
+  // where the sequences and heads are few, so that more blocks walk shorter chains
+  const long long wide_blocks = 1LL * n_seqs * H * ((DV + 63) / 64);
+  const bool narrow = wide_blocks < 2LL * ei_compute_units();
+  const int cols = narrow ? 16 : 64;
+  const dim3 grid(n_seqs, H, (DV + cols - 1) / cols);
   const size_t ss = static_cast<size_t>(split_stride), rs = static_cast<size_t>(row_stride);
-#define EI_LA(TI, R)                                                                           \
-  la_scan_kernel<TI, R><<<grid, kCols * kGroups, 0, stream>>>(                                 \
+#define EI_LA(TI, R, COLS)                                                                     \
+  la_scan_kernel<TI, R, COLS><<<grid, kThreads, 0, stream>>>(                                  \
       static_cast<const TI*>(proj), nsplit, ss, rs, decay, state, state, seq_in, seq_out,      \
       seq_count, seq_row0, o_raw, H, DK, DV)
 #define EI_LA_T(TI)                                 \
   do {                                              \
-    if (DK <= 32) EI_LA(TI, 8);                     \
-    else if (DK <= 64) EI_LA(TI, 16);               \
-    else if (DK <= 128) EI_LA(TI, 32);              \
-    else EI_LA(TI, 64);                             \
+    if (narrow) {                                   \
+      if (DK <= 64) EI_LA(TI, 4, 16);               \
+      else if (DK <= 128) EI_LA(TI, 8, 16);         \
+      else EI_LA(TI, 16, 16);                       \
+    } else if (DK <= 32) EI_LA(TI, 8, 64);          \
+    else if (DK <= 64) EI_LA(TI, 16, 64);           \
+    else if (DK <= 128) EI_LA(TI, 32, 64);          \
+    else EI_LA(TI, 64, 64);                         \
   } while (0)
   if (proj_dtype == EI_F32) EI_LA_T(float);
   else if (proj_dtype == EI_BF16) EI_LA_T(bf16_t);

@@ -83,6 +83,144 @@ __global__ void stream_norm_kernel(float* __restrict__ residual, const TD* __res
     dst[i] = ei::from_f32<TO>(((values[i] - mean) * inv) * w_next[i] + (b_next ? b_next[i] : 0.f));
 }
 
+using ei::Vec4;
+
+// Four neighbouring elements of a row as the sum of its slices, in slice order; eight loads are
+// issued before the first sum, so that a row costs one trip to memory per eight slices.
+template <typename TD>
+__device__ __forceinline__ void sliced4(const TD* p, int nsplit, size_t split_stride, float (&x)[4]) {
+  x[0] = x[1] = x[2] = x[3] = 0.f;
+  for (int s0 = 0; s0 < nsplit; s0 += 8) {
+    float v[8][4];
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (s0 + u < nsplit) Vec4<TD>::load(p + (s0 + u) * split_stride, v[u]);
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (s0 + u < nsplit) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) x[i] += v[u][i];
+      }
+  }
+}
+
+// mean and 1 / sqrt(variance + eps) of a row that the block's threads hold in registers
+// (CHUNKS quads a thread; quads beyond the row hold zeros and are told by `live`).
+template <int CHUNKS>
+__device__ __forceinline__ void held_moments(const float (&x)[CHUNKS][4], const bool (&live)[CHUNKS],
+                                             int H, int centred, float eps, float* scratch,
+                                             float& mean, float& inv) {
+  mean = 0.f;
+  if (centred) {
+    float sum = 0.f;
+#pragma unroll
+    for (int k = 0; k < CHUNKS; ++k)
+      if (live[k]) sum += (x[k][0] + x[k][1]) + (x[k][2] + x[k][3]);
+    mean = ei::block_sum(sum, scratch) / static_cast<float>(H);
+  }
+  float squares = 0.f;
+#pragma unroll
+  for (int k = 0; k < CHUNKS; ++k)
+    if (live[k]) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) squares += (x[k][i] - mean) * (x[k][i] - mean);
+    }
+  inv = 1.0f / sqrtf(ei::block_sum(squares, scratch) / static_cast<float>(H) + eps);
+}
+
+// stream_norm_kernel for widths that are a multiple of 4: 16-byte accesses, the row kept in
+// registers, up to 1024 threads a row so that few rows still have many loads in flight.
+template <typename TD, typename TO, int CHUNKS>
+__global__ void stream_norm_vec_kernel(float* __restrict__ residual, const TD* __restrict__ delta,
+                                       int nsplit, size_t split_stride,
+                                       const float* __restrict__ delta_bias,
+                                       const int32_t* __restrict__ rows,
+                                       const float* __restrict__ w_after,
+                                       const float* __restrict__ b_after,
+                                       const float* __restrict__ w_next,
+                                       const float* __restrict__ b_next, float eps, int centred,
+                                       TO* __restrict__ out, int H, int write_residual) {
+  __shared__ float scratch[16];
+  const int row = blockIdx.x;
+  const int src = rows ? rows[row] : row;
+  const int quads = H / 4;
+  if (src < 0) {
+    if (out) {
+      const float zero[4] = {0.f, 0.f, 0.f, 0.f};
+      for (int qd = threadIdx.x; qd < quads; qd += blockDim.x)
+        Vec4<TO>::store(out + static_cast<size_t>(row) * H + qd * 4, zero);
+    }
+    return;
+  }
+  float* res = residual + static_cast<size_t>(src) * H;
+  bool live[CHUNKS];
+  float y[CHUNKS][4];
+#pragma unroll
+  for (int k = 0; k < CHUNKS; ++k) {
+    const int qd = threadIdx.x + k * blockDim.x;
+    live[k] = qd < quads;
+    y[k][0] = y[k][1] = y[k][2] = y[k][3] = 0.f;
+    if (live[k]) Vec4<float>::load(res + qd * 4, y[k]);
+  }
+  if (delta) {
+    float x[CHUNKS][4];
+#pragma unroll
+    for (int k = 0; k < CHUNKS; ++k) {
+      const int qd = threadIdx.x + k * blockDim.x;
+      x[k][0] = x[k][1] = x[k][2] = x[k][3] = 0.f;
+      if (live[k]) {
+        sliced4(delta + static_cast<size_t>(src) * H + qd * 4, nsplit, split_stride, x[k]);
+        if (delta_bias) {
+          float b[4];
+          Vec4<float>::load(delta_bias + qd * 4, b);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) x[k][i] += b[i];
+        }
+      }
+    }
+    if (w_after) {
+      float mean, inv;
+      held_moments<CHUNKS>(x, live, H, centred, eps, scratch, mean, inv);
+#pragma unroll
+      for (int k = 0; k < CHUNKS; ++k) {
+        const int qd = threadIdx.x + k * blockDim.x;
+        if (live[k]) {
+          float w[4], b[4] = {0.f, 0.f, 0.f, 0.f};
+          Vec4<float>::load(w_after + qd * 4, w);
+          if (b_after) Vec4<float>::load(b_after + qd * 4, b);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) x[k][i] = ((x[k][i] - mean) * inv) * w[i] + b[i];
+        }
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < CHUNKS; ++k) {
+      const int qd = threadIdx.x + k * blockDim.x;
+      if (live[k]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) y[k][i] += x[k][i];
+        if (write_residual) Vec4<float>::store(res + qd * 4, y[k]);
+      }
+    }
+  }
+  if (!out) return;
+  float mean, inv;
+  held_moments<CHUNKS>(y, live, H, centred, eps, scratch, mean, inv);
+  TO* dst = out + static_cast<size_t>(row) * H;
+#pragma unroll
+  for (int k = 0; k < CHUNKS; ++k) {
+    const int qd = threadIdx.x + k * blockDim.x;
+    if (live[k]) {
+      float w[4], b[4] = {0.f, 0.f, 0.f, 0.f}, z[4];
+      Vec4<float>::load(w_next + qd * 4, w);
+      if (b_next) Vec4<float>::load(b_next + qd * 4, b);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) z[i] = ((y[k][i] - mean) * inv) * w[i] + b[i];
+      Vec4<TO>::store(dst + qd * 4, z);
+    }
+  }
+}
+
 constexpr int kMaxBranches = 4;
 
 struct Branches {
@@ -126,6 +264,69 @@ __global__ void norm_mean_kernel(Branches branches, int n, float eps, float* __r
   for (int i = threadIdx.x; i < H; i += blockDim.x) out[base + i] = total[i] * share;
 }
 
+// norm_mean_kernel for widths that are a multiple of 4 (and slices that lie a multiple of 4
+// apart): 16-byte accesses, rows and running sums kept in registers.
+template <int CHUNKS>
+__global__ void norm_mean_vec_kernel(Branches branches, int n, float eps, float* __restrict__ out,
+                                     int H) {
+  __shared__ float scratch[16];
+  const size_t base = static_cast<size_t>(blockIdx.x) * H;
+  const int quads = H / 4;
+  float total[CHUNKS][4];
+#pragma unroll
+  for (int k = 0; k < CHUNKS; ++k) total[k][0] = total[k][1] = total[k][2] = total[k][3] = 0.f;
+  for (int b = 0; b < n; ++b) {
+    const bool narrow = branches.dtype[b] == EI_BF16;
+    const size_t stride = static_cast<size_t>(branches.split_stride[b]);
+    float x[CHUNKS][4];
+    float squares = 0.f;
+#pragma unroll
+    for (int k = 0; k < CHUNKS; ++k) {
+      const int qd = threadIdx.x + k * blockDim.x;
+      x[k][0] = x[k][1] = x[k][2] = x[k][3] = 0.f;
+      if (qd < quads) {
+        if (narrow)
+          sliced4(static_cast<const bf16_t*>(branches.rows[b]) + base + qd * 4, branches.nsplit[b],
+                  stride, x[k]);
+        else
+          sliced4(static_cast<const float*>(branches.rows[b]) + base + qd * 4, branches.nsplit[b],
+                  stride, x[k]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) squares += x[k][i] * x[k][i];
+      }
+    }
+    const float inv = 1.0f / sqrtf(ei::block_sum(squares, scratch) / static_cast<float>(H) + eps);
+#pragma unroll
+    for (int k = 0; k < CHUNKS; ++k) {
+      const int qd = threadIdx.x + k * blockDim.x;
+      if (qd < quads) {
+        float w[4];
+        Vec4<float>::load(branches.weight[b] + qd * 4, w);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) total[k][i] += (x[k][i] * inv) * w[i];
+      }
+    }
+  }
+  const float share = 1.0f / static_cast<float>(n);
+#pragma unroll
+  for (int k = 0; k < CHUNKS; ++k) {
+    const int qd = threadIdx.x + k * blockDim.x;
+    if (qd < quads) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) total[k][i] *= share;
+      Vec4<float>::store(out + base + qd * 4, total[k]);
+    }
+  }
+}
+
+// Threads a row of the register-held forms: up to 1024 for few rows, so that many loads are in
+// flight; 256 for many rows, so that several rows share a compute unit.
+int vec_threads(int N, int quads) {
+  const int most = N >= 512 && quads <= 4 * 256 ? 256 : 1024;
+  int threads = (quads + EI_WAVE - 1) / EI_WAVE * EI_WAVE;
+  return threads > most ? most : threads;
+}
+
 int row_threads(int H) { return H >= 4096 ? 512 : (H >= 1024 ? 256 : (H >= 256 ? 128 : 64)); }
 
 }  // namespace
@@ -151,16 +352,30 @@ extern "C" int ei_stream_norm(float* residual, const void* delta, int delta_dtyp
   const size_t ss = static_cast<size_t>(split_stride);
   if (!delta) delta_dtype = EI_F32;
   if (!out) out_dtype = EI_F32;
-#define EI_SN(TD, TO)                                                                          \
-  stream_norm_kernel<TD, TO><<<N, threads, lds, stream>>>(                                     \
+  const bool vec = H % 4 == 0 && (!delta || ss % 4 == 0) && H <= 16384;
+  const int vthreads = vec_threads(N, H / 4);
+  const int chunks = vec ? (H / 4 + vthreads - 1) / vthreads : 0;      // 1..4
+#define EI_SN_VEC(TD, TO, C)                                                                   \
+  stream_norm_vec_kernel<TD, TO, C><<<N, vthreads, 0, stream>>>(                               \
       residual, static_cast<const TD*>(delta), nsplit, ss, delta_bias, rows, w_after, b_after, \
       w_next, b_next, eps, centred, static_cast<TO*>(out), H, write_residual)
+#define EI_SN(TD, TO)                                                                          \
+  do {                                                                                         \
+    if (chunks == 1) EI_SN_VEC(TD, TO, 1);                                                     \
+    else if (chunks == 2) EI_SN_VEC(TD, TO, 2);                                                \
+    else if (chunks == 3 || chunks == 4) EI_SN_VEC(TD, TO, 4);                                 \
+    else                                                                                       \
+      stream_norm_kernel<TD, TO><<<N, threads, lds, stream>>>(                                 \
+          residual, static_cast<const TD*>(delta), nsplit, ss, delta_bias, rows, w_after,      \
+          b_after, w_next, b_next, eps, centred, static_cast<TO*>(out), H, write_residual);    \
+  } while (0)
   if (delta_dtype == EI_F32 && out_dtype == EI_F32) EI_SN(float, float);
   else if (delta_dtype == EI_F32 && out_dtype == EI_BF16) EI_SN(float, bf16_t);
   else if (delta_dtype == EI_BF16 && out_dtype == EI_BF16) EI_SN(bf16_t, bf16_t);
   else if (delta_dtype == EI_BF16 && out_dtype == EI_F32) EI_SN(bf16_t, float);
   else EI_REQUIRE(false, "stream_norm: unknown dtype");
 #undef EI_SN
+#undef EI_SN_VEC
   EI_LAUNCH_CHECK();
 }
 
@@ -185,6 +400,16 @@ extern "C" int ei_norm_mean(const void* const* x, const int* nsplit, const long 
   }
   const int threads = row_threads(H);
   const size_t lds = static_cast<size_t>(H) * 2 * sizeof(float);
-  norm_mean_kernel<<<N, threads, lds, stream>>>(branches, n, eps, out, H);
+  bool vec = H % 4 == 0 && H <= 16384;
+  for (int b = 0; b < n; ++b)
+    vec = vec && split_stride[b] % 4 == 0 && reinterpret_cast<uintptr_t>(x[b]) % 16 == 0;
+  const int vthreads = vec_threads(N, H / 4);
+  const int chunks = vec ? (H / 4 + vthreads - 1) / vthreads : 0;
+  if (chunks == 1) norm_mean_vec_kernel<1><<<N, vthreads, 0, stream>>>(branches, n, eps, out, H);
+  else if (chunks == 2) norm_mean_vec_kernel<2><<<N, vthreads, 0, stream>>>(branches, n, eps, out, H);
+  else if (chunks == 3 || chunks == 4)
+    norm_mean_vec_kernel<4><<<N, vthreads, 0, stream>>>(branches, n, eps, out, H);
+  else
+    norm_mean_kernel<<<N, threads, lds, stream>>>(branches, n, eps, out, H);
   EI_LAUNCH_CHECK();
 }

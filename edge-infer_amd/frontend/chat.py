@@ -21,7 +21,7 @@ import time
 from pathlib import Path
 
 MODEL_TYPES = ("qwen3_bf16", "qwen3_fp32", "tirurax_bf16", "tirurax_fp32", "zadenex_bf16",
-               "zadenex_fp32", "vafepel_bf16", "vafepel_fp32")
+               "zadenex_fp32", "vafepel_bf16", "vafepel_fp32", "gopuzen_bf16", "gopuzen_fp32")
 
 
 def load_tokenizer(model_path):
@@ -147,7 +147,7 @@ def build_parser() -> argparse.ArgumentParser:
                         help="local folder with config.json, safetensors and (for text) tokenizer.json")
     parser.add_argument("--model_type", type=str, default="qwen3_bf16", choices=MODEL_TYPES,
                         help="<family>_bf16, or <family>_fp32 for the true 32-bit path; the "
-                             "family (qwen3, tirurax, zadenex, vafepel) must be the one config.json names")
+                             "family (qwen3, tirurax, zadenex, vafepel, gopuzen) must be the one config.json names")
     parser.add_argument("--device", type=str, default="cuda", choices=["cuda"],
                         help="execution device (this library runs on the GPU only)")
     parser.add_argument("--system_prompt", type=str, default="You are a helpful AI assistant.")

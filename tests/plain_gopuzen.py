@@ -155,9 +155,13 @@ def attention_mixer(h, tensors, prefix, mixer, positions, shared):
     else:
         k, v = shared
     mask = mixer.get("mask")
-    if mask:
+    if mask and mask.get("pool") is not None:
         out = pooled_window_attention(q, k, v, float(mixer["scale"]), int(mask["size"]),
                                       int(mask["pool"]))
+    elif mask:
+        size = int(mask["size"])
+        out = softmax_attention(q, k, v, float(mixer["scale"]),
+                                lambda i: list(range(max(0, i - size + 1), i + 1)))
     else:
         out = softmax_attention(q, k, v, float(mixer["scale"]), lambda i: list(range(i + 1)))
     gate = sigmoid(linear(h, tensors[prefix + "g"]))              # [T, H]
@@ -216,10 +220,25 @@ def route(h, tensors, prefix, router):
     return chosen, torch.gather(scores, 1, chosen), scores
 
 
-def routed_feed_forward(h, tensors, prefix, mlp):
+def choice_margins(h, tensors, prefix, router):
+    """For every row the gap between the last chosen and the first unchosen choice score,
+    relative to the larger of the two: a rounding that is larger may choose otherwise (what a
+    rounding does to a score grows with the score)."""
+    scores = torch.softmax(linear(h, tensors[prefix + "router"]), dim=-1)
+    choice = torch.sort(scores + f64(tensors[prefix + "correction"]), dim=-1, descending=True).values
+    top = int(router["top"])
+    if top >= choice.shape[1]:
+        return torch.full((choice.shape[0],), float("inf"), dtype=F64)
+    larger = torch.maximum(choice[:, top - 1].abs(), choice[:, top].abs()).clamp_min(1e-30)
+    return (choice[:, top - 1] - choice[:, top]) / larger
+
+
+def routed_feed_forward(h, tensors, prefix, mlp, margins=None):
     router = mlp["router"]
     experts = int(router["experts"])
     chosen, weights, _ = route(h, tensors, prefix, router)
+    if margins is not None:
+        margins.append(choice_margins(h, tensors, prefix, router))
     h = f64(h)
     out = torch.zeros_like(h)
     for t in range(h.shape[0]):
@@ -234,9 +253,10 @@ def routed_feed_forward(h, tensors, prefix, mlp):
 
 
 # ---------------------------------------------------------------------------- the model
-def forward(cfg, tensors, tokens, layer_outputs=None):
+def forward(cfg, tensors, tokens, layer_outputs=None, margins=None):
     """Logits [T, vocab] of one sequence of token ids from position 0.  `layer_outputs`: a
-    list that receives the stream after every layer."""
+    list that receives the stream after every layer; `margins`: a list that receives, for
+    every routed feed-forward, the rows' choice margins."""
     eps = float(cfg["norm"]["eps"])
     tokens = torch.as_tensor(tokens, dtype=torch.int64)
     positions = torch.arange(tokens.shape[0])
@@ -264,9 +284,24 @@ def forward(cfg, tensors, tokens, layer_outputs=None):
             if mlp["kind"] == "dense":
                 f = dense_feed_forward(h, tensors, name + "mlp.")
             else:
-                f = routed_feed_forward(h, tensors, name + "mlp.", mlp)
+                f = routed_feed_forward(h, tensors, name + "mlp.", mlp, margins)
             x = x + norm("norm2b", f) * f64(tensors[name + "ls2"])
         if layer_outputs is not None:
             layer_outputs.append(x.clone())
     x = layer_norm(x, tensors["final.norm"], tensors["final.norm.b"], eps)
     return linear(x, tensors["head"])
+
+
+def clear_rows(cfg, tensors, tokens, margin, carry=True):
+    """(logits, mask of the positions whose logits no routing decision closer than `margin`
+    can have touched).  `carry`: a close call at a position also touches every later one (the
+    caches and states carry it on)."""
+    margins = []
+    logits = forward(cfg, tensors, tokens, margins=margins)
+    clear = torch.ones(logits.shape[0], dtype=torch.bool)
+    for rows in margins:
+        clear &= rows >= margin
+    if carry and not bool(clear.all()):
+        first = int((~clear).nonzero()[0])
+        clear[first:] = False
+    return logits, clear
