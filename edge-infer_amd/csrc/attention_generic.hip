@@ -18,7 +18,9 @@
 // row and head: the output is multiplied by sigmoid(gate)), `pool` (with a window w: besides the
 // tokens of its window a query at p sees entry b of a second paged cache, which holds one key and
 // value for every block of `pool` positions, if b pool + pool - 1 <= p - w; tokens and blocks
-// share one softmax).
+// share one softmax), `pool_only` (the tokens are left out: the kernel takes the pooled entries
+// alone and leaves every row's unnormalised sums, maximum and sum of weights in part_o and
+// part_ml, slice 0 of one, for a kernel that takes them in as one more slice of its own softmax).
 // operators/src/cuda/execution.cu:137-179, runtime/src/qwen.cpp:374-402,
 // split merge: operators/src/cuda/kernels/gather_fa_variable.cu:14-118.
 #include "common.h"
@@ -43,7 +45,8 @@ attn_generic_kernel(const T* __restrict__ q, const T* __restrict__ k_pages,
                     const float* __restrict__ slopes, const float* __restrict__ sinks,
                     float scale, int n_splits, int KH, int values_in_keys,
                     const float* __restrict__ gate, int pool, const T* __restrict__ pool_k,
-                    const T* __restrict__ pool_v, const int32_t* __restrict__ pool_table) {
+                    const T* __restrict__ pool_v, const int32_t* __restrict__ pool_table,
+                    int pool_only) {
   extern __shared__ float lds[];
   const int DQ = KH * D;                  // width of a query row and of a key as it is met
   float* Qs = lds;                        // [kRows][DQ]
@@ -175,7 +178,7 @@ attn_generic_kernel(const T* __restrict__ q, const T* __restrict__ k_pages,
     const int p_begin = lo_page + split * per;
     const int p_end = min(lo_page + (split + 1) * per, hi_page + 1);
     const int chunks_per_page = EI_PAGE / BC;
-    for (int p = p_begin; p < p_end; ++p) {
+    for (int p = p_begin; p < p_end && !pool_only; ++p) {
       const int phys = page_table[static_cast<size_t>(seq) * table_width + p];
       if (phys < 0) continue;  // a page the window has released: every key in it is masked
       const T* kp = k_pages + (static_cast<size_t>(phys) * nkv + g) * EI_PAGE * D;
@@ -211,7 +214,7 @@ attn_generic_kernel(const T* __restrict__ q, const T* __restrict__ k_pages,
   }
 
   if (!row_valid) return;
-  if (sinks && split == 0) {
+  if (sinks && split == 0 && !pool_only) {
     // the sink is one more term of the denominator: exp(sink), on the row's running scale
     const float sink = sinks[head];
     const float m_new = fmaxf(m_r, sink);
@@ -221,7 +224,7 @@ attn_generic_kernel(const T* __restrict__ q, const T* __restrict__ k_pages,
     for (int k = 0; k < kAcc; ++k) acc[k] *= alpha;
     m_r = m_new;
   }
-  if (n_splits == 1) {
+  if (n_splits == 1 && !pool_only) {
     float inv = l_r > 0.f ? 1.f / l_r : 0.f;
     if (gate) inv *= 1.0f / (1.0f + expf(-gate[static_cast<size_t>(row) * nq + head]));
     T* dst = out + (static_cast<size_t>(row) * nq + head) * DV;
@@ -292,7 +295,8 @@ extern "C" int ei_attention(const void* q, const void* k_pages, const void* v_pa
                             int D, int DV, int window, int chunk, const float* slopes,
                             const float* sinks, float scale, int n_splits, int key_heads,
                             int values_in_keys, const float* gate, int pool, const void* pool_k,
-                            const void* pool_v, const int32_t* pool_table, hipStream_t stream) {
+                            const void* pool_v, const int32_t* pool_table, int pool_only,
+                            hipStream_t stream) {
   EI_REQUIRE(n_items > 0 && N > 0 && nq > 0 && nkv > 0, "attention: sizes must be positive");
   EI_REQUIRE(nq % nkv == 0, "attention: query heads must be a multiple of kv heads");
   EI_REQUIRE(key_heads == 1 || key_heads == nkv,
@@ -307,7 +311,9 @@ extern "C" int ei_attention(const void* q, const void* k_pages, const void* v_pa
                  page_table && table_width > 0,
              "attention: null pointer");
   EI_REQUIRE(n_splits >= 1 && n_splits <= 64, "attention: splits must be between 1 and 64");
-  EI_REQUIRE(n_splits == 1 || (part_o && part_ml), "attention: split scratch missing");
+  EI_REQUIRE((n_splits == 1 && !pool_only) || (part_o && part_ml), "attention: split scratch missing");
+  EI_REQUIRE(!pool_only || (pool > 0 && n_splits == 1 && !gate),
+             "attention: the pooled entries alone are taken in one slice, without a gate");
   EI_REQUIRE(window >= 0, "attention: negative window");
   EI_REQUIRE(pool >= 0 && (pool == 0 || (window > 0 && pool_k && pool_v && pool_table &&
                                          key_heads == 1 && !values_in_keys)),
@@ -342,14 +348,14 @@ extern "C" int ei_attention(const void* q, const void* k_pages, const void* v_pa
         static_cast<const float*>(v_pages), item_seq, item_row0, item_npos, row_pos, page_table,
         table_width, static_cast<float*>(out), part_o, part_ml, nq, nkv, D, DV, Gb, head_blocks,
         BC, window, chunk, slopes, sinks, scale, n_splits, key_heads, values_in_keys, gate, pool,
-        static_cast<const float*>(pool_k), static_cast<const float*>(pool_v), pool_table);
+        static_cast<const float*>(pool_k), static_cast<const float*>(pool_v), pool_table, pool_only);
   } else if (dtype == EI_BF16) {
     attn_generic_kernel<bf16_t><<<grid, kThreads, lds, stream>>>(
         static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pages),
         static_cast<const bf16_t*>(v_pages), item_seq, item_row0, item_npos, row_pos, page_table,
         table_width, static_cast<bf16_t*>(out), part_o, part_ml, nq, nkv, D, DV, Gb, head_blocks,
         BC, window, chunk, slopes, sinks, scale, n_splits, key_heads, values_in_keys, gate, pool,
-        static_cast<const bf16_t*>(pool_k), static_cast<const bf16_t*>(pool_v), pool_table);
+        static_cast<const bf16_t*>(pool_k), static_cast<const bf16_t*>(pool_v), pool_table, pool_only);
   } else {
     EI_REQUIRE(false, "attention: unknown dtype");
   }

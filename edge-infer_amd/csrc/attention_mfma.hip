@@ -29,10 +29,18 @@ constexpr float kLowest = -1.0e30f;
 // ones are compiled without any of this): `chunk` > 0: a query at p sees key t only if
 // t / chunk == p / chunk; `slopes` (per query head, or null): slope * (p - t) is taken off the
 // scaled score; `sinks` (per query head, or null): exp(sink) joins the softmax's denominator.
+// `pool_o`, `pool_ml` (or null): what another kernel has gathered for every (row, head) from keys
+// of another source (the pooled blocks before a window): float32 sums of weighted values
+// [rows, nq, D] and (maximum, sum of weights) [rows, nq, 2] in natural units; they join the
+// row's softmax as one more slice.  `gate` (float32 [rows, nq], or null): the output of a row
+// and head is multiplied by sigmoid(gate).
 struct AttnExtra {
   int chunk;
   const float* slopes;
   const float* sinks;
+  const float* pool_o;
+  const float* pool_ml;
+  const float* gate;
 };
 
 __device__ __forceinline__ float bf16_lo(uint32_t u) { return __uint_as_float(u << 16); }
@@ -493,6 +501,8 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
   // running maximum and sum per row here, its output tile in the page buffers
   __shared__ float handed_lds[KW == 2 ? kPrefillWaves / 2 : 1][2][kWideRows];
   __shared__ __attribute__((aligned(16))) float other_lds[KW == 2 ? kPrefillWaves : 1][kWideRows];
+  // (EXT) what the other source's sums of a row are scaled by
+  __shared__ __attribute__((aligned(16))) float pool_lds[EXT ? kPrefillWaves : 1][kWideRows];
   static_assert(KW == 1 || (kPrefillWaves / 2) * (D / 32) * 16 * EI_WAVE * sizeof(float) <=
                                sizeof(bf16_t) * kPageBuffers * 2 * PBUF,
                 "the handed-over output tiles fit the page buffers");
@@ -854,8 +864,26 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
       m_run = m_new;
     }
   }
+  float pool_scale = 0.f;      // (EXT) what the other source's sums are scaled by, before 1 / l
+  if constexpr (EXT) {
+    if (extra.pool_ml && kw == 0 && pw * kWideRows + n32 < npos) {
+      // the other source's slice of this lane's row: one more (maximum, sum) to take in
+      const size_t slot = static_cast<size_t>(row0 + pw * kWideRows + n32) * nq + head;
+      const float m_p = extra.pool_ml[2 * slot] * 1.4426950408889634f;
+      const float l_p = extra.pool_ml[2 * slot + 1];
+      if (l_p > 0.f) {
+        const float m_new = fmaxf(m_run, m_p);
+        const float fold = __builtin_amdgcn_exp2f(m_run - m_new);
+        pool_scale = __builtin_amdgcn_exp2f(m_p - m_new);
+        l_wave = l_wave * fold + l_p * pool_scale;
+        sink_fold *= fold;
+        m_run = m_new;
+      }
+    }
+  }
   float own_factor = l_wave > 0.f ? sink_fold / l_wave : 0.f;   // what this wave's output is scaled by
   float other_factor = 0.f;                               // and the handed-over one
+  float pool_factor = l_wave > 0.f ? pool_scale / l_wave : 0.f;
   if constexpr (KW == 2) {
     // The wave of the second half of every page's keys hands its state to the wave of the
     // first: o = (o_0 2^(m_0 - m) + o_1 2^(m_1 - m)) / (l_0 2^(m_0 - m) + l_1 2^(m_1 - m)).
@@ -883,11 +911,22 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
       const float inv = l > 0.f ? 1.f / l : 0.f;
       own_factor = sink_fold * f_own * inv;
       other_factor = f_other * inv;
+      pool_factor = pool_scale * f_own * inv;
+    }
+  }
+  if constexpr (EXT) {
+    if (extra.gate && kw == 0 && pw * kWideRows + n32 < npos) {
+      const float gate = extra.gate[static_cast<size_t>(row0 + pw * kWideRows + n32) * nq + head];
+      const float open = 1.0f / (1.0f + expf(-gate));
+      own_factor *= open;
+      other_factor *= open;
+      pool_factor *= open;
     }
   }
   if (half == 0) {
     factor_lds[wave][n32] = own_factor;
     if constexpr (KW == 2) other_lds[wave][n32] = other_factor;
+    if constexpr (EXT) pool_lds[wave][n32] = pool_factor;
   }
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
@@ -902,6 +941,11 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
         const float4 add4 = *reinterpret_cast<const float4*>(&other_lds[wave][8 * i + 4 * half]);
         add[0] = add4.x; add[1] = add4.y; add[2] = add4.z; add[3] = add4.w;
       }
+      float pooled[4] = {0.f, 0.f, 0.f, 0.f};
+      if constexpr (EXT) {
+        const float4 p4 = *reinterpret_cast<const float4*>(&pool_lds[wave][8 * i + 4 * half]);
+        pooled[0] = p4.x; pooled[1] = p4.y; pooled[2] = p4.z; pooled[3] = p4.w;
+      }
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int orow = pw * kWideRows + 8 * i + 4 * half + r;
@@ -915,6 +959,11 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
             o = fmaf(tile_lds[(((wave % (HB * NG)) * DB + db) * 16 + 4 * i + r) * EI_WAVE + lane],
                      add[r], o);
           }
+          if constexpr (EXT) {
+            if (extra.pool_o && pooled[r] != 0.f)
+              o = fmaf(extra.pool_o[(static_cast<size_t>(row0 + orow) * nq + head) * D + db * 32 + n32],
+                       pooled[r], o);
+          }
           dst[db * 32 + n32] = ei::from_f32<bf16_t>(o);
         }
       }
@@ -926,10 +975,15 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
 }
 
 // One wave per (row, head): o = sum_s o_s e^{m_s - m} / sum_s l_s e^{m_s - m}.
+// pool_o, pool_ml (or null): one more slice a (row, head), from another source of keys; gate (or
+// null): the result is multiplied by sigmoid(gate[row, head]).
 __global__ void attn_merge_kernel(const float* __restrict__ part_o,
                                   const float* __restrict__ part_ml,
                                   const int32_t* __restrict__ row_seq, bf16_t* __restrict__ out,
-                                  int nq, int D, int n_splits, int total) {
+                                  int nq, int D, int n_splits, int total,
+                                  const float* __restrict__ pool_o,
+                                  const float* __restrict__ pool_ml,
+                                  const float* __restrict__ gate) {
   const int wave = (blockIdx.x * blockDim.x + threadIdx.x) / EI_WAVE;
   const int lane = threadIdx.x % EI_WAVE;
   if (wave >= total) return;
@@ -961,8 +1015,22 @@ __global__ void attn_merge_kernel(const float* __restrict__ part_o,
           m = m_new;
         }
     }
+    if (pool_ml) {
+      const float2 st = reinterpret_cast<const float2*>(pool_ml)[wave];
+      if (st.y > 0.f) {
+        const float2 ov = d < D ? *reinterpret_cast<const float2*>(pool_o + static_cast<size_t>(wave) * D + d)
+                                : float2{0.f, 0.f};
+        const float m_new = fmaxf(m, st.x);
+        const float keep = expf(m - m_new), add = expf(st.x - m_new);
+        l = l * keep + st.y * add;
+        o0 = o0 * keep + ov.x * add;
+        o1 = o1 * keep + ov.y * add;
+        m = m_new;
+      }
+    }
     if (d < D) {
-      const float inv = l > 0.f ? 1.f / l : 0.f;
+      float inv = l > 0.f ? 1.f / l : 0.f;
+      if (gate) inv *= 1.0f / (1.0f + expf(-gate[wave]));
       bf16_t* dst = out + static_cast<size_t>(wave) * D + d;
       dst[0] = ei::from_f32<bf16_t>(o0 * inv);
       dst[1] = ei::from_f32<bf16_t>(o1 * inv);
@@ -1108,10 +1176,13 @@ extern "C" int ei_attention_prefill_mfma_ext(
     const int32_t* item_row0, const int32_t* item_npos, int n_items, const int32_t* row_pos,
     const int32_t* page_table, int table_width, void* out, int nq, int nkv, int D, int window,
     float scale, int key_ways, int pair_items, int chunk, const float* slopes,
-    const float* sinks, hipStream_t stream) {
+    const float* sinks, const float* pool_o, const float* pool_ml, const float* gate,
+    hipStream_t stream) {
   EI_REQUIRE(chunk >= 0, "attention_prefill: negative chunk");
   EI_REQUIRE(scale > 0.f, "attention_prefill: the scale must be positive");
-  const AttnExtra extra{chunk, slopes, sinks};
+  EI_REQUIRE((pool_o == nullptr) == (pool_ml == nullptr),
+             "attention_prefill: the other source's sums and their weights come together");
+  const AttnExtra extra{chunk, slopes, sinks, pool_o, pool_ml, gate};
   return prefill_launch(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items, row_pos,
                         page_table, table_width, out, nq, nkv, D, window, scale, key_ways,
                         pair_items, &extra, stream);
@@ -1130,6 +1201,11 @@ static int decode_launch(const void* q, const void* k_pages, const void* v_pages
                          const DecodePrep* prep, hipStream_t stream,
                          const AttnExtra* extra = nullptr) {
   EI_REQUIRE(!(prep && extra), "attention_decode: the fused projection has no extended form");
+  EI_REQUIRE(!extra || n_splits > 1 || !(extra->pool_ml || extra->gate),
+             "attention_decode: a second source of keys and the gate are taken in by the merge "
+             "of at least two slices");
+  EI_REQUIRE(!extra || (extra->pool_o == nullptr) == (extra->pool_ml == nullptr),
+             "attention_decode: the other source's sums and their weights come together");
   EI_REQUIRE(rows > 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attention_decode: bad head counts");
   EI_REQUIRE(waves == 4 || waves == 8 || waves == 16,
              "attention_decode: a block has 4, 8 or 16 waves");
@@ -1161,7 +1237,7 @@ static int decode_launch(const void* q, const void* k_pages, const void* v_pages
   const bf16_t* vv = static_cast<const bf16_t*>(v_pages);
   bf16_t* oo = static_cast<bf16_t*>(out);
   const DecodePrep none{};
-  const AttnExtra plain{0, nullptr, nullptr};
+  const AttnExtra plain{0, nullptr, nullptr, nullptr, nullptr, nullptr};
 #define EI_DECODE(DD, GG)                                                                     \
   do {                                                                                        \
     if (prep)                                                                                 \
@@ -1204,8 +1280,9 @@ static int decode_launch(const void* q, const void* k_pages, const void* v_pages
     const int total = rows * nq;
     const int threads = 256;
     const int blocks = (total * EI_WAVE + threads - 1) / threads;
-    attn_merge_kernel<<<blocks, threads, 0, stream>>>(part_o, part_ml, row_seq, oo, nq, D,
-                                                      n_splits, total);
+    attn_merge_kernel<<<blocks, threads, 0, stream>>>(
+        part_o, part_ml, row_seq, oo, nq, D, n_splits, total, extra ? extra->pool_o : nullptr,
+        extra ? extra->pool_ml : nullptr, extra ? extra->gate : nullptr);
   }
   EI_LAUNCH_CHECK();
 }
@@ -1239,9 +1316,10 @@ extern "C" int ei_attention_decode_mfma_ext(const void* q, const void* k_pages,
                                             int window, float scale, int n_splits, int waves,
                                             int heads, const int32_t* longest, int chunk,
                                             const float* slopes, const float* sinks,
-                                            hipStream_t stream) {
+                                            const float* pool_o, const float* pool_ml,
+                                            const float* gate, hipStream_t stream) {
   EI_REQUIRE(chunk >= 0, "attention_decode: negative chunk");
-  const AttnExtra extra{chunk, slopes, sinks};
+  const AttnExtra extra{chunk, slopes, sinks, pool_o, pool_ml, gate};
   return decode_launch(q, k_pages, v_pages, row_pos, row_seq, page_table, table_width, out,
                        part_o, part_ml, rows, nq, nkv, D, window, scale, n_splits, waves, heads,
                        longest, nullptr, stream, &extra);

@@ -123,7 +123,7 @@ _SIGNATURES = {
         "ei_attention": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
                          c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
                          c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float,
-                         c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p],
+                         c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p],
         "ei_pool_store": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                           c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
     },
@@ -171,11 +171,11 @@ _SIGNATURES = {
         "ei_attention_prefill_mfma_ext": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                           c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p,
                                           c_int, c_int, c_int, c_int, c_float, c_int, c_int,
-                                          c_int, c_void_p, c_void_p, c_void_p],
+                                          c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
         "ei_attention_decode_mfma_ext": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                          c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
                                          c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int,
-                                         c_void_p, c_int, c_void_p, c_void_p, c_void_p],
+                                         c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
         "ei_attention_decode_mfma_fused": [c_void_p, c_int, c_longlong, c_void_p, c_void_p, c_float,
                                            c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                            c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
@@ -593,7 +593,7 @@ def attention(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items, row_
               page_table, out, n_heads, n_kv_heads, head_dim, window=None, scale=None,
               n_splits=1, part_o=None, part_ml=None, value_dim=None, chunk=None, slopes=None,
               sinks=None, key_heads=1, values_in_keys=False, gate=None, pool=None,
-              pool_k=None, pool_v=None, pool_table=None) -> None:
+              pool_k=None, pool_v=None, pool_table=None, pool_only=False) -> None:
     """Generic causal attention over the paged cache (see attention_generic.hip).
     value_dim: head size of the values and of `out` (None: head_dim); chunk: a query sees only
     the keys of its own block of that many positions; slopes, sinks: float32 [n_heads], the
@@ -604,7 +604,10 @@ def attention(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items, row_
     rows and `v_pages` is not read.  gate: float32 [rows, heads]; the output of a row and
     head is multiplied by sigmoid(gate).  pool: P (needs a window): a query also sees the
     entries of the pooled cache (`pool_k`, `pool_v`: pages shaped like the tokens' pages, found
-    through `pool_table`) whose blocks of P positions lie wholly before its window."""
+    through `pool_table`) whose blocks of P positions lie wholly before its window.
+    pool_only: the tokens are left out; `out` is not written, and part_o [rows, heads,
+    value_dim] and part_ml [rows, heads, 2] receive every row's unnormalised sums over the
+    pooled entries, the largest score and the sum of weights (n_splits 1)."""
     lib = library("attention_generic")
     n = q.shape[0]
     value_dim = head_dim if value_dim is None else int(value_dim)
@@ -634,7 +637,9 @@ def attention(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items, row_
     for name, per_head in (("slopes", slopes), ("sinks", sinks)):
         if per_head is not None and per_head.numel() != n_heads:
             raise KernelError(f"attention: {name} must have one value per query head")
-    if n_splits > 1:
+    if pool_only and (not pool or n_splits != 1 or gate is not None):
+        raise KernelError("attention: the pooled entries alone are taken in one slice")
+    if n_splits > 1 or pool_only:
         need_o = n * n_heads * n_splits * value_dim
         if part_o is None or part_ml is None or part_o.numel() < need_o \
                 or part_ml.numel() < n * n_heads * n_splits * 2:
@@ -662,7 +667,8 @@ def attention(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items, row_
         key_heads, int(bool(values_in_keys)),
         None if gate is None else _gpu(gate, "gate", torch.float32), int(pool or 0),
         _gpu(pool_k, "pool_k") if pool else None, _gpu(pool_v, "pool_v") if pool else None,
-        _gpu(pool_table, "pool_table", torch.int32) if pool else None, _stream())
+        _gpu(pool_table, "pool_table", torch.int32) if pool else None, int(bool(pool_only)),
+        _stream())
     _check(lib, status, "attention")
 
 
@@ -1062,7 +1068,8 @@ def attention_prefill_mfma_positions(group: int, key_ways: int = 1) -> int:
 def attention_prefill_mfma(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items, row_pos,
                            page_table, out, n_heads, n_kv_heads, head_dim, window=None,
                            scale=None, key_ways=1, pair_items=True, largest_item=None,
-                           chunk=None, slopes=None, sinks=None) -> None:
+                           chunk=None, slopes=None, sinks=None, pool_o=None, pool_ml=None,
+                           gate=None) -> None:
     """bfloat16 prefill attention on the matrix cores; an item holds up to
     `attention_prefill_mfma_positions(group, key_ways)` positions of one sequence.
     pair_items: with enough items a block may take item i and then item n_items - 1 - i
@@ -1099,21 +1106,35 @@ def attention_prefill_mfma(q, k_pages, v_pages, item_seq, item_row0, item_npos, 
         _gpu(page_table, "page_table", torch.int32), page_table.shape[-1],
         _gpu(out, "out", torch.bfloat16), n_heads, n_kv_heads, head_dim, int(window or 0),
         float(scale), int(key_ways), int(bool(pair_items)))
-    if chunk or slopes is not None or sinks is not None:
+    if chunk or slopes is not None or sinks is not None or pool_o is not None or gate is not None:
         status = lib.ei_attention_prefill_mfma_ext(*common, *_attention_extras(
-            chunk, slopes, sinks, n_heads), _stream())
+            chunk, slopes, sinks, n_heads, n, head_dim, pool_o, pool_ml, gate), _stream())
     else:
         status = lib.ei_attention_prefill_mfma(*common, _stream())
     _check(lib, status, "attention_prefill")
 
 
-def _attention_extras(chunk, slopes, sinks, n_heads):
-    """(chunk, slopes pointer, sinks pointer) for the extended forms of the matrix-core kernels."""
+def _attention_extras(chunk, slopes, sinks, n_heads, rows=0, head_dim=0, pool_o=None,
+                      pool_ml=None, gate=None):
+    """(chunk, slopes, sinks, pool_o, pool_ml, gate pointers) for the extended forms of the
+    matrix-core kernels.  pool_o float32 [rows * heads * head_dim] and pool_ml [rows * heads *
+    2]: what `attention(..., pool_only=True)` left for every row and head, taken in as one more
+    slice of the softmax; gate float32 [rows, heads]: the output is multiplied by its sigmoid."""
     for name, per_head in (("slopes", slopes), ("sinks", sinks)):
         if per_head is not None and per_head.numel() != n_heads:
             raise KernelError(f"attention: {name} must have one value per query head")
-    return (int(chunk or 0), None if slopes is None else _gpu(slopes, "slopes", torch.float32),
-            None if sinks is None else _gpu(sinks, "sinks", torch.float32))
+    if (pool_o is None) != (pool_ml is None):
+        raise KernelError("attention: the pooled sums and their weights come together")
+    if pool_o is not None and (pool_o.numel() < rows * n_heads * head_dim
+                               or pool_ml.numel() < rows * n_heads * 2):
+        raise KernelError("attention: the pooled sums are too small for these rows")
+    if gate is not None and gate.numel() < rows * n_heads:
+        raise KernelError("attention: the gate must be float32 [rows, heads]")
+
+    def f32(tensor, name):
+        return None if tensor is None else _gpu(tensor, name, torch.float32)
+    return (int(chunk or 0), f32(slopes, "slopes"), f32(sinks, "sinks"), f32(pool_o, "pool_o"),
+            f32(pool_ml, "pool_ml"), f32(gate, "gate"))
 
 
 class DecodeProjection:
@@ -1131,7 +1152,7 @@ class DecodeProjection:
 def attention_decode_mfma(q, k_pages, v_pages, row_pos, row_seq, page_table, out, n_heads,
                           n_kv_heads, head_dim, window=None, scale=None, n_splits=1, part_o=None,
                           part_ml=None, waves=4, longest=None, heads=0, chunk=None, slopes=None,
-                          sinks=None) -> None:
+                          sinks=None, pool_o=None, pool_ml=None, gate=None) -> None:
     """bfloat16 decode attention on the matrix cores: one query row per sequence.  `waves`
     (4, 8 or 16) of a block share its key range tile by tile; more suit fewer sequences (few
     blocks), whose ranges then need fewer slices or none.  `heads` (a power of two, or 0 for
@@ -1145,7 +1166,11 @@ def attention_decode_mfma(q, k_pages, v_pages, row_pos, row_seq, page_table, out
     lib = library("attention_mfma")
     n = out.shape[0]
     fused = isinstance(q, DecodeProjection)
-    extended = bool(chunk) or slopes is not None or sinks is not None
+    extended = (bool(chunk) or slopes is not None or sinks is not None or pool_o is not None
+                or gate is not None)
+    if (pool_o is not None or gate is not None) and n_splits < 2:
+        raise KernelError("attention_decode: pooled sums and the gate are taken in by the merge "
+                          "of at least two slices")
     if fused and extended:
         raise KernelError("attention_decode: the fused projection has no extended form")
     if tuple(out.shape) != (n, n_heads * head_dim) or (not fused and tuple(q.shape) != tuple(out.shape)):
@@ -1200,7 +1225,7 @@ def attention_decode_mfma(q, k_pages, v_pages, row_pos, row_seq, page_table, out
         None if longest is None else _gpu(longest, "longest", torch.int32))
     if extended:
         status = lib.ei_attention_decode_mfma_ext(*common, *_attention_extras(
-            chunk, slopes, sinks, n_heads), _stream())
+            chunk, slopes, sinks, n_heads, q.shape[0], head_dim, pool_o, pool_ml, gate), _stream())
     else:
         status = lib.ei_attention_decode_mfma(*common, _stream())
     _check(lib, status, "attention_decode")

@@ -160,13 +160,15 @@ class Attention:
         step."""
         group = spec.n_heads // max(1, spec.n_kv_heads)
         fast = (dtype == torch.bfloat16 and spec.v_dim == spec.head_dim and MATRIX_CORE_ATTENTION
-                and not spec.talking_heads and spec.pool is None and spec.output_gate != "head"
+                and not spec.talking_heads
                 and lib.attention_decode_mfma_supported(spec.head_dim, group))
         kernels = "attention_mfma" if fast else "attention_generic"
         if cls.wide_keys(spec, dtype):
             kernels = "attention_wide"
-        return ("rope_store", kernels, *(("head_ops",) if spec.talking_heads else ()),
-                *Linear.kernel_libraries(dtype))
+        # (the pooled blocks are stored, and beside the matrix-core kernels also gathered, by
+        # kernels of the generic library)
+        return ("rope_store", kernels, *(("attention_generic",) if spec.pool is not None else ()),
+                *(("head_ops",) if spec.talking_heads else ()), *Linear.kernel_libraries(dtype))
 
     @classmethod
     def wide_keys(cls, spec, dtype) -> bool:
@@ -306,8 +308,10 @@ class Attention:
         # as the keys; every other case runs the generic kernel
         self.matrix_cores = (dtype == torch.bfloat16 and spec.v_dim == spec.head_dim and
                             MATRIX_CORE_ATTENTION and self.talk is None and
-                            spec.pool is None and not self.head_gate and
                             lib.attention_decode_mfma_supported(spec.head_dim, self.group))
+        # beside the matrix-core kernels the pooled blocks are gathered by the generic kernel
+        # (they are few: one for `pool` tokens) and taken in as one more slice of the softmax
+        self.pooled_aside = self.matrix_cores and spec.pool is not None
         # chunk, slopes, sink: what the kernels take beyond a window
         self.wide = self.wide_keys(spec, dtype)
         self.extras = dict(chunk=spec.chunk, slopes=self.slopes, sinks=self.sinks)
@@ -357,10 +361,28 @@ class Attention:
     @property
     def plan_key(self):
         """Attention parts with equal keys plan the same sections."""
-        return ("attention", self.positions_per_item(), self.group, self.spec.n_kv_heads, self.wide)
+        return ("attention", self.positions_per_item(), self.group, self.spec.n_kv_heads, self.wide,
+                self.pooled_aside)
 
     def _items_section(self, key_ways: int = 1):
         return f"attention.items{self.positions_per_item(key_ways)}"
+
+    def _aside_size(self) -> int:
+        """Positions of an item of the generic kernel, which gathers the pooled blocks beside
+        the matrix-core kernels."""
+        return lib.attention_positions_per_item(self.group)
+
+    @staticmethod
+    def _prompt_items(plan, size: int):
+        """Every sequence's rows cut into items of `size`, the ones with the longest key range
+        first, as [3, items]: sequence, first row, positions."""
+        items = []
+        for index, seq in enumerate(plan.seqs):
+            for p0 in range(0, seq.count, size):
+                npos = min(size, seq.count - p0)
+                items.append((-(seq.start + p0 + npos), index, seq.row0 + p0, npos))
+        items.sort()
+        return np.asarray([item[1:] for item in items], dtype=np.int32).T.copy()
 
     def plan_step(self, plan):
         """The work items of this step's attention kernels, as one int32 section [3, items]:
@@ -370,15 +392,13 @@ class Attention:
         if plan.decode:
             return {"attention.decode_items": _decode_items(plan.n_seqs, plan.n_live_seqs)}
         key_ways = self.prefill_key_ways([seq.count for seq in plan.seqs])
-        size = self.positions_per_item(key_ways)
-        items = []
-        for index, seq in enumerate(plan.seqs):
-            for p0 in range(0, seq.count, size):
-                npos = min(size, seq.count - p0)
-                items.append((-(seq.start + p0 + npos), index, seq.row0 + p0, npos))
-        items.sort()
-        return {self._items_section(key_ways): np.asarray([item[1:] for item in items],
-                                                          dtype=np.int32).T.copy()}
+        sections = {self._items_section(key_ways):
+                    self._prompt_items(plan, self.positions_per_item(key_ways))}
+        if self.pooled_aside:
+            name = f"attention.items{self._aside_size()}"
+            if name not in sections:
+                sections[name] = self._prompt_items(plan, self._aside_size())
+        return sections
 
     @staticmethod
     def _items(ctx, name):
@@ -467,7 +487,7 @@ class Attention:
         # (the kernel that norms and stores the whole projection adds its bias as well)
         qkv, bias = (self.qkv.forward(ctx, x, "attn.qkv", bias_later=True) if self.whole_store
                      else (self.qkv.forward(ctx, x, "attn.qkv"), None))
-        gate, pooled = None, {}
+        gate, pooled, aside = None, {}, {}
         if self.general:
             q = ctx.buffer("attn.q", (n, spec.q_width))
             v_first, v_mode = None, 0
@@ -501,6 +521,21 @@ class Attention:
                 lib.pool_store(k_pages, v_pages, meta.row_pos, meta.row_seq, page_table,
                                pool_table, pool_k, pool_v, n, spec.pool)
                 pooled = dict(pool=spec.pool, pool_k=pool_k, pool_v=pool_v, pool_table=pool_table)
+                if self.pooled_aside:
+                    # every row's sums over the pooled blocks it sees, for the matrix-core
+                    # kernels to take in as one more slice
+                    pool_o = ctx.buffer("attn.pool_o", (n * spec.n_heads * spec.v_dim,), torch.float32)
+                    pool_ml = ctx.buffer("attn.pool_ml", (n * spec.n_heads * 2,), torch.float32)
+                    items = self._items(ctx, "attention.decode_items" if ctx.decode
+                                        else f"attention.items{self._aside_size()}")
+                    # (in this mode the kernel writes the sums only; `q` stands where the
+                    # output's shape is asked for)
+                    lib.attention(q, k_pages, v_pages, items[0], items[1], items[2], items[3],
+                                  meta.row_pos, meta.row_seq, page_table, q, spec.n_heads,
+                                  spec.n_kv_heads, spec.head_dim, window=spec.window,
+                                  scale=self.scale, part_o=pool_o, part_ml=pool_ml,
+                                  value_dim=spec.v_dim, pool_only=True, **pooled)
+                    aside = dict(pool_o=pool_o, pool_ml=pool_ml)
         elif (ctx.decode and self.matrix_cores and FUSED_DECODE and qkv.dim() == 3
                 and qkv.dtype == torch.float32 and not self.whole_store and not self.has_extras):
             # the decode kernel norms, rotates and stores for its rows itself: one launch less
@@ -530,6 +565,8 @@ class Attention:
         part_o = part_ml = None
         if ctx.decode:
             splits, waves, heads = self._decode_launch_for(ctx.n_seqs, ctx.context_bound)
+            if self.matrix_cores and (aside or gate is not None):
+                splits = max(2, splits)      # the merge of slices takes the other source and the gate in
             if splits > 1:
                 part_o = ctx.buffer("attn.part_o", (n * spec.n_heads * splits * spec.v_dim,),
                                     torch.float32)
@@ -541,7 +578,7 @@ class Attention:
                                           spec.head_dim, window=spec.window, scale=self.scale,
                                           n_splits=splits, part_o=part_o, part_ml=part_ml,
                                           waves=waves, longest=meta.longest, heads=heads,
-                                          **self.extras)
+                                          gate=gate, **aside, **self.extras)
             else:
                 item_seq, item_row0, item_npos, n_items = self._items(ctx, "attention.decode_items")
                 if self.wide:
@@ -572,7 +609,7 @@ class Attention:
                                            spec.n_kv_heads, spec.head_dim, window=spec.window,
                                            scale=self.scale, key_ways=key_ways,
                                            pair_items=len({(seq.start, seq.count) for seq in ctx.sequences}) == 1,
-                                           largest_item=largest, **self.extras)
+                                           largest_item=largest, gate=gate, **aside, **self.extras)
             elif self.wide:
                 lib.attention_wide(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items,
                                    meta.row_pos, meta.row_seq, page_table, out, spec.n_heads,
@@ -586,7 +623,8 @@ class Attention:
                               scale=self.scale, **more)
         if spec.output_gate and not self.head_gate:
             lib.gate_rows(qkv, self.gate_column, out)
-        ctx.release(qkv, None if isinstance(q, lib.DecodeProjection) else q, part_o, part_ml, gate)
+        ctx.release(qkv, None if isinstance(q, lib.DecodeProjection) else q, part_o, part_ml, gate,
+                    aside.get("pool_o"), aside.get("pool_ml"))
         delta = self.o.forward(ctx, out, "attn.o", bias_later=bias_later)
         ctx.release(out)
         return delta
