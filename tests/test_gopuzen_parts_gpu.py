@@ -38,14 +38,16 @@ def test_layer_norm_in_its_three_places(width, slices):
     summed = delta if slices == 0 else delta.double().sum(0)
     w1, b1, w2, b2 = (exact((width,), g) for _ in range(4))
     bias = exact((width,), g, 0.3)
-    # before a sublayer: the delta is added, rows 5, 0, 3 are normed
+    # before a sublayer: rows 5, 0, 3 take their delta and are normed (-1: a padding row); the
+    # other rows are not touched
     res = residual.clone().to(DEV)
     pick = torch.tensor([5, 0, -1, 3], dtype=torch.int32, device=DEV)
     out = torch.empty(4, width, device=DEV)
     lib.stream_norm(res, delta.to(DEV), out, w_next=w2.to(DEV), b_next=b2.to(DEV), eps=EPS,
                     centred=True, rows=pick)
     added = residual.double() + summed
-    assert_close_f32(res, added, "stream after the addition")
+    assert_close_f32(res[[5, 0, 3]], added[[5, 0, 3]], "stream after the addition")
+    assert torch.equal(res[[1, 2, 4, 6]].cpu(), residual[[1, 2, 4, 6]])
     want = plain.layer_norm(added[[5, 0, 3]], w2, b2, EPS)
     assert_close_f32(out[[0, 1, 3]], want, "gathered rows")
     assert out[2].abs().max().item() == 0.0
