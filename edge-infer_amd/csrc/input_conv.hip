@@ -1,9 +1,9 @@
 // A short causal convolution over time that is added to what it reads: for every channel c of
 // a row at step index t of its sequence,
 //
-//   out_t[c] = h_t[c] + sum_j w[c, j] * h_(t - T + 1 + j)[c],    j = 0 .. T - 1,
+//   out_t[c] = h_t[c] + sum_j w[j, c] * h_(t - T + 1 + j)[c],    j = 0 .. T - 1,
 //
-// with rows before the sequence's start being zero.  The last T - 1 inputs of a sequence are
+// (the filter lies tap by tap, [T, W], so that neighbouring channels' weights are neighbours) with rows before the sequence's start being zero.  The last T - 1 inputs of a sequence are
 // its state: a float32 table with two versions of every sequence's row, [tables rows]
 // [parts][T - 1][W]; a step reads the row `seq_in` names and writes the whole part `part` of
 // the row `seq_out` names, so a prompt may arrive whole, in portions of any size or token by
@@ -53,8 +53,10 @@ input_conv_kernel(const T* __restrict__ h, const float* __restrict__ w,
       float x[VEC];
       if (at >= 0) load_row(h + static_cast<size_t>(row0 + at) * W + c, x);
       else load_state(old + static_cast<size_t>(tail + at) * W + c, x);
+      float wj[VEC];
+      load_state(w + static_cast<size_t>(j) * W + c, wj);
 #pragma unroll
-      for (int i = 0; i < VEC; ++i) acc[i] += w[static_cast<size_t>(c + i) * taps + j] * x[i];
+      for (int i = 0; i < VEC; ++i) acc[i] += wj[i] * x[i];
     }
     if constexpr (VEC == 8) ei::VecN<T, 8>::store(out + static_cast<size_t>(row) * W + c, acc);
     else out[static_cast<size_t>(row) * W + c] = ei::from_f32<T>(acc[0]);
@@ -81,7 +83,7 @@ input_conv_kernel(const T* __restrict__ h, const float* __restrict__ w,
 
 }  // namespace
 
-// h, out: [N, W] of `dtype` (out may not be h: later rows read earlier ones); w: [W, taps]
+// h, out: [N, W] of `dtype` (out may not be h: later rows read earlier ones); w: [taps, W]
 // float32; state: float32 rows of parts * (taps - 1) * W (null when taps is 1).
 extern "C" int ei_input_conv(const void* h, int dtype, const float* w, float* state, int part,
                              int parts, int taps, const int32_t* row_pos, const int32_t* row_seq,
@@ -95,7 +97,7 @@ extern "C" int ei_input_conv(const void* h, int dtype, const float* w, float* st
   EI_REQUIRE(row_pos && row_seq && seq_start && seq_count && seq_row0, "input_conv: row metadata missing");
   EI_REQUIRE(taps == 1 || (state && seq_in && seq_out), "input_conv: state missing");
   const auto aligned16 = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
-  const bool vec = W % 8 == 0 && aligned16(h) && aligned16(out) && aligned16(state);
+  const bool vec = W % 8 == 0 && aligned16(h) && aligned16(out) && aligned16(state) && aligned16(w);
   const int per = vec ? 8 : 1;
   const size_t items = (static_cast<size_t>(N) + static_cast<size_t>(n_seqs) * (taps - 1)) * (W / per);
   const unsigned blocks = static_cast<unsigned>((items + 255) / 256);

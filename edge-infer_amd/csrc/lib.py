@@ -89,7 +89,9 @@ _SIGNATURES = {
     "linear_attention": {
         "ei_la_scan": [c_void_p, c_int, c_int, c_longlong, c_longlong, c_void_p, c_void_p,
                        c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
-                       c_int, c_void_p],
+                       c_int, c_int, c_void_p],
+        "ei_la_activate": [c_void_p, c_int, c_int, c_longlong, c_longlong, c_void_p, c_int, c_int,
+                           c_void_p],
         "ei_la_out": [c_void_p, c_void_p, c_int, c_int, c_longlong, c_longlong, c_longlong,
                       c_void_p, c_float, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
     },
@@ -1546,15 +1548,15 @@ def norm_mean(branches, weights, eps: float, out: torch.Tensor) -> None:
 def input_conv(h, weight, state, part: int, parts: int, row_pos, row_seq, seq_in, seq_out,
                seq_start, seq_count, seq_row0, out) -> None:
     """out [n, w] = h + conv(h): a causal convolution over the rows of every sequence with
-    the filter weight [w, taps] (float32), the inputs before the step's rows taken from part
+    the filter weight [taps, w] (float32, tap by tap), the inputs before the step's rows taken from part
     `part` of the sequence's state row (float32 rows of parts * (taps - 1) * w, two versions:
     `seq_in` names the row read, `seq_out` the row whose part is written anew).  state None
     with one tap."""
     lib = library("input_conv")
     n, width = h.shape
-    taps = weight.shape[1]
+    taps = weight.shape[0]
     n_seqs = seq_count.numel()
-    if tuple(weight.shape) != (width, taps) or tuple(out.shape) != (n, width) or out.dtype != h.dtype:
+    if tuple(weight.shape) != (taps, width) or tuple(out.shape) != (n, width) or out.dtype != h.dtype:
         raise KernelError("input_conv: shapes do not fit")
     if out.data_ptr() == h.data_ptr():
         raise KernelError("input_conv: the result needs a buffer of its own")
@@ -1582,13 +1584,30 @@ def la_state_floats(heads: int, key_dim: int, value_dim: int) -> int:
     return heads * key_dim * value_dim
 
 
+def la_activate(proj, act) -> None:
+    """act [n, w] float32 = silu of the first w columns of proj's rows ([n, g] or float32 slices
+    [s, n, g]): q, k and v of linear attention, activated once for every block of the scan."""
+    lib = library("linear_attention")
+    n, width = act.shape
+    stride = proj.shape[-1]
+    nsplit, split_stride = _splits(proj, n, stride, "proj")
+    if stride < width:
+        raise KernelError("la_activate: the rows are narrower than what is asked of them")
+    status = lib.ei_la_activate(_gpu(proj, "proj"), _code(proj, "proj"), nsplit, split_stride,
+                                stride, _gpu(act, "act", torch.float32), n, width, _stream())
+    _check(lib, status, "la_activate")
+
+
 def la_scan(proj, decay, state, seq_in, seq_out, seq_count, seq_row0, o_raw, heads, key_dim,
-            value_dim) -> None:
+            value_dim, activated: bool = False) -> None:
     """The recurrence of linear attention with a decay per head over the rows of every
     sequence: proj rows [q | k | v | ...] ([n, g] or float32 slices [s, n, g]), silu on all
     three, S_t = decay_h S_(t-1) + k_t v_t^T, o_raw [n, heads * value_dim] float32 = S_t^T q_t.
-    state: float32 rows of heads * key_dim * value_dim, two versions (`seq_in`, `seq_out`)."""
+    state: float32 rows of heads * key_dim * value_dim, two versions (`seq_in`, `seq_out`).
+    activated: the rows hold q, k and v as `la_activate` left them, and silu is not taken again."""
     lib = library("linear_attention")
+    if activated and proj.dtype != torch.float32:
+        raise KernelError("la_scan: activated rows are float32")
     n = o_raw.shape[0]
     stride = proj.shape[-1]
     nsplit, split_stride = _splits(proj, n, stride, "proj")
@@ -1606,7 +1625,8 @@ def la_scan(proj, decay, state, seq_in, seq_out, seq_count, seq_row0, o_raw, hea
         _gpu(decay, "decay", torch.float32), _gpu(state, "state", torch.float32),
         _gpu(seq_in, "seq_in", torch.int32), _gpu(seq_out, "seq_out", torch.int32),
         _gpu(seq_count, "seq_count", torch.int32), _gpu(seq_row0, "seq_row0", torch.int32),
-        _gpu(o_raw, "o_raw", torch.float32), n_seqs, heads, key_dim, value_dim, _stream())
+        _gpu(o_raw, "o_raw", torch.float32), n_seqs, heads, key_dim, value_dim,
+        int(bool(activated)), _stream())
     _check(lib, status, "la_scan")
 
 

@@ -28,9 +28,13 @@ __device__ __forceinline__ float silu_f32(float x) { return x / (1.0f + expf(-x)
 
 // A block a (sequence, head, COLS columns of S).  Thread (c, g): column c, rows g R .. g R + R - 1
 // (R a multiple of 4; the 256 / COLS groups g hold G R >= DK rows; rows beyond DK hold zeros).
-// A tile of 16 tokens' q, k and v lies in LDS while its tokens are walked; the next tile's
-// values are asked of global memory before the walk and wait in registers.
-template <typename TI, int R, int COLS>
+// A tile of 16 tokens' q, k and v lies in LDS while its tokens are walked; with AHEAD the next
+// tile's values are asked of global memory before the walk and wait in registers (launches of
+// few blocks, which live on how soon a tile is there; launches that fill the chip lose more by
+// the registers than they gain).  ACT: the rows hold raw projections and silu is taken here;
+// else they hold q, k and v as `la_activate` left them (a prompt's many tokens: every block of
+// a head would take the same silu of q and k again).
+template <typename TI, int R, int COLS, bool AHEAD, bool ACT>
 __global__ void __launch_bounds__(kThreads)
 la_scan_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride, size_t row_stride,
                const float* __restrict__ decay, const float* state_in_table, float* state_out_table,
@@ -92,22 +96,25 @@ la_scan_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride, siz
                            nsplit, split_stride);
     }
   };
-  fetch(0);
+  if constexpr (AHEAD) fetch(0);
   for (int tile0 = 0; tile0 < count; tile0 += kTile) {
     const int nt = min(kTile, count - tile0);
+    if constexpr (!AHEAD) fetch(tile0);
 #pragma unroll
     for (int u = 0; u < QK_PER; ++u) {
       const int idx = t + u * kThreads;
-      qs[idx / DKP][idx % DKP] = silu_f32(q_next[u]);
-      ks[idx / DKP][idx % DKP] = silu_f32(k_next[u]);
+      qs[idx / DKP][idx % DKP] = ACT ? silu_f32(q_next[u]) : q_next[u];
+      ks[idx / DKP][idx % DKP] = ACT ? silu_f32(k_next[u]) : k_next[u];
     }
 #pragma unroll
     for (int u = 0; u < V_PER; ++u) {
       const int idx = t + u * kThreads;
-      if (idx < kTile * COLS) vs[idx / COLS][idx % COLS] = silu_f32(v_next[u]);
+      if (idx < kTile * COLS) vs[idx / COLS][idx % COLS] = ACT ? silu_f32(v_next[u]) : v_next[u];
     }
     __syncthreads();
-    if (tile0 + kTile < count) fetch(tile0 + kTile);
+    if constexpr (AHEAD) {
+      if (tile0 + kTile < count) fetch(tile0 + kTile);
+    }
     for (int tt = 0; tt < nt; ++tt) {
       const float vv = vs[tt][c];
       const float4* kq = reinterpret_cast<const float4*>(&ks[tt][g * R]);
@@ -146,6 +153,17 @@ la_scan_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride, siz
   }
 }
 
+// act [N, width] float32 = silu(sum of the slices of the first `width` columns of proj's rows).
+template <typename TI>
+__global__ void la_activate_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride,
+                                   size_t row_stride, float* __restrict__ act, size_t total,
+                                   int width) {
+  const size_t index = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (index >= total) return;
+  const size_t row = index / width, col = index % width;
+  act[index] = silu_f32(sliced(proj + row * row_stride + col, nsplit, split_stride));
+}
+
 // A block a row: out = o / sqrt(mean(o^2) + eps) * w * sigmoid(g), g the columns of the
 // projection from `gate_at` on (the sum of its float32 slices).
 template <typename TI, typename TO>
@@ -181,7 +199,7 @@ extern "C" int ei_la_scan(const void* proj, int proj_dtype, int nsplit, long lon
                           long long row_stride, const float* decay, float* state,
                           const int32_t* seq_in, const int32_t* seq_out, const int32_t* seq_count,
                           const int32_t* seq_row0, float* o_raw, int n_seqs, int H, int DK, int DV,
-                          hipStream_t stream) {
+                          int activated, hipStream_t stream) {
   EI_REQUIRE(proj && decay && state && seq_in && seq_out && seq_count && seq_row0 && o_raw,
              "la_scan: null pointer");
   EI_REQUIRE(n_seqs > 0 && H > 0 && DK >= 1 && DK <= 256 && DV >= 1 && nsplit >= 1,
@@ -191,30 +209,57 @@ extern "C" int ei_la_scan(const void* proj, int proj_dtype, int nsplit, long lon
   // 64 columns a block where that fills the chip; 16 (and a quarter of the rows a thread)
   // where the sequences and heads are few, so that more blocks walk shorter chains
   const long long wide_blocks = 1LL * n_seqs * H * ((DV + 63) / 64);
-  const bool narrow = wide_blocks < 2LL * ei_compute_units();
+  const bool narrow = wide_blocks < ei_compute_units();
   const int cols = narrow ? 16 : 64;
   const dim3 grid(n_seqs, H, (DV + cols - 1) / cols);
   const size_t ss = static_cast<size_t>(split_stride), rs = static_cast<size_t>(row_stride);
-#define EI_LA(TI, R, COLS)                                                                     \
-  la_scan_kernel<TI, R, COLS><<<grid, kThreads, 0, stream>>>(                                  \
-      static_cast<const TI*>(proj), nsplit, ss, rs, decay, state, state, seq_in, seq_out,      \
-      seq_count, seq_row0, o_raw, H, DK, DV)
-#define EI_LA_T(TI)                                 \
-  do {                                              \
-    if (narrow) {                                   \
-      if (DK <= 64) EI_LA(TI, 4, 16);               \
-      else if (DK <= 128) EI_LA(TI, 8, 16);         \
-      else EI_LA(TI, 16, 16);                       \
-    } else if (DK <= 32) EI_LA(TI, 8, 64);          \
-    else if (DK <= 64) EI_LA(TI, 16, 64);           \
-    else if (DK <= 128) EI_LA(TI, 32, 64);          \
-    else EI_LA(TI, 64, 64);                         \
+#define EI_LA(TI, R, COLS, AHEAD)                                                              \
+  do {                                                                                         \
+    if (activated)                                                                             \
+      la_scan_kernel<TI, R, COLS, AHEAD, false><<<grid, kThreads, 0, stream>>>(                \
+          static_cast<const TI*>(proj), nsplit, ss, rs, decay, state, state, seq_in, seq_out,  \
+          seq_count, seq_row0, o_raw, H, DK, DV);                                              \
+    else                                                                                       \
+      la_scan_kernel<TI, R, COLS, AHEAD, true><<<grid, kThreads, 0, stream>>>(                 \
+          static_cast<const TI*>(proj), nsplit, ss, rs, decay, state, state, seq_in, seq_out,  \
+          seq_count, seq_row0, o_raw, H, DK, DV);                                              \
+  } while (0)
+#define EI_LA_T(TI)                                       \
+  do {                                                    \
+    if (narrow) {                                         \
+      if (DK <= 64) EI_LA(TI, 4, 16, true);               \
+      else if (DK <= 128) EI_LA(TI, 8, 16, true);         \
+      else EI_LA(TI, 16, 16, true);                       \
+    } else if (DK <= 32) EI_LA(TI, 8, 64, false);         \
+    else if (DK <= 64) EI_LA(TI, 16, 64, false);          \
+    else if (DK <= 128) EI_LA(TI, 32, 64, false);         \
+    else EI_LA(TI, 64, 64, false);                        \
   } while (0)
   if (proj_dtype == EI_F32) EI_LA_T(float);
   else if (proj_dtype == EI_BF16) EI_LA_T(bf16_t);
   else EI_REQUIRE(false, "la_scan: unknown dtype");
 #undef EI_LA_T
 #undef EI_LA
+  EI_LAUNCH_CHECK();
+}
+
+// act: float32 [N, width] = silu of the first `width` columns of proj's rows (q, k and v).
+extern "C" int ei_la_activate(const void* proj, int proj_dtype, int nsplit, long long split_stride,
+                              long long row_stride, float* act, int N, int width,
+                              hipStream_t stream) {
+  EI_REQUIRE(proj && act && N > 0 && width > 0 && nsplit >= 1 && row_stride >= width,
+             "la_activate: bad arguments");
+  const size_t total = static_cast<size_t>(N) * width;
+  const unsigned blocks = static_cast<unsigned>((total + 255) / 256);
+  const size_t ss = static_cast<size_t>(split_stride), rs = static_cast<size_t>(row_stride);
+  if (proj_dtype == EI_F32)
+    la_activate_kernel<float><<<blocks, 256, 0, stream>>>(static_cast<const float*>(proj), nsplit, ss,
+                                                          rs, act, total, width);
+  else if (proj_dtype == EI_BF16)
+    la_activate_kernel<bf16_t><<<blocks, 256, 0, stream>>>(static_cast<const bf16_t*>(proj), nsplit,
+                                                           ss, rs, act, total, width);
+  else
+    EI_REQUIRE(false, "la_activate: unknown dtype");
   EI_LAUNCH_CHECK();
 }
 

@@ -342,9 +342,10 @@ class SandwichBlock:
         self.taps = int(getattr(layer_spec, "input_conv", 0))
         self.conv1 = self.conv2 = None
         if self.taps:
-            self.conv1 = params["conv1.weight"].to(device=device, dtype=torch.float32).contiguous()
+            # (kept tap by tap, [taps, width]: neighbouring channels' weights are neighbours)
+            self.conv1 = params["conv1.weight"].to(device=device, dtype=torch.float32).t().contiguous()
             if self.ffn is not None:
-                self.conv2 = params["conv2.weight"].to(device=device, dtype=torch.float32).contiguous()
+                self.conv2 = params["conv2.weight"].to(device=device, dtype=torch.float32).t().contiguous()
 
     def _convolved(self, ctx, h, entry, part):
         """h + conv(h) for sublayer `part` (0: the mixer, 1: the feed-forward)."""

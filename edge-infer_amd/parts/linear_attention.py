@@ -26,6 +26,8 @@ from .linear import Linear
 
 
 class LinearAttention:
+    ACTIVATE_ROWS = 64       # from so many rows of a prompt step on, q, k and v are activated aside
+
     @property
     def capture_safe(self):
         """Only this library's kernels, nothing allocated per step, what varies read from the
@@ -86,8 +88,17 @@ class LinearAttention:
         state = ctx.cache.state(entry.cache)                 # [2 (slots + 1), state floats]
         proj = self.proj.forward(ctx, x, "la.proj")
         o_raw = ctx.buffer("la.o_raw", (n, spec.v_width), torch.float32)
-        lib.la_scan(proj, self.decay, state, meta.seq_state_in, meta.seq_state_out, meta.seq_count,
-                    meta.seq_row0, o_raw, spec.n_heads, spec.key_dim, spec.value_dim)
+        rows, activated = proj, False
+        if not ctx.decode and n >= self.ACTIVATE_ROWS:
+            # many tokens a sequence: silu of q, k and v once, not once a block of the scan
+            rows = ctx.buffer("la.act", (n, self.gate_column), torch.float32)
+            lib.la_activate(proj, rows)
+            activated = True
+        lib.la_scan(rows, self.decay, state, meta.seq_state_in, meta.seq_state_out, meta.seq_count,
+                    meta.seq_row0, o_raw, spec.n_heads, spec.key_dim, spec.value_dim,
+                    activated=activated)
+        if activated:
+            ctx.release(rows)
         gated = ctx.buffer("la.gated", (n, spec.v_width))
         lib.la_out(o_raw, proj, self.gate_column, self.out_norm, spec.norm_eps, meta.row_seq, gated)
         ctx.release(o_raw, proj)

@@ -127,7 +127,8 @@ class ConvRig:
             return torch.tensor(values, dtype=torch.int32, device=DEV)
         h = torch.cat([x for _, x in pieces]).to(DEV).to(dtype).contiguous()
         out = torch.empty_like(h)
-        lib.input_conv(h, weight.to(DEV), self.state if self.taps > 1 else None, part, self.parts,
+        lib.input_conv(h, weight.t().contiguous().to(DEV), self.state if self.taps > 1 else None,
+                       part, self.parts,
                        i32(row_pos), i32(row_seq), i32(seq_in), i32(seq_out), i32(start),
                        i32(count), i32(row0), out)
         return out.float().cpu()
@@ -208,10 +209,15 @@ def test_linear_attention_recurrence(heads, key_dim, value_dim, seqs):
         for _, _, n in taken:
             row0.append(at)
             at += n
-        lib.la_scan(rows, decay.to(DEV), state,
+        scanned, activated = rows, total % 2 == 0
+        if activated:       # (q, k and v activated aside, as a prompt step of many rows does)
+            scanned = torch.empty(total, heads * (2 * key_dim + value_dim), device=DEV)
+            lib.la_activate(rows, scanned)
+        lib.la_scan(scanned, decay.to(DEV), state,
                     i32([version[s] * (seqs + 1) + s for s, _, _ in taken]),
                     i32([(1 - version[s]) * (seqs + 1) + s for s, _, _ in taken]),
-                    i32([n for _, _, n in taken]), i32(row0), o_raw, heads, key_dim, value_dim)
+                    i32([n for _, _, n in taken]), i32(row0), o_raw, heads, key_dim, value_dim,
+                    activated=activated)
         out = torch.empty(total, heads * value_dim, device=DEV)
         lib.la_out(o_raw, rows, 2 * heads * key_dim + heads * value_dim, norm_w.to(DEV), EPS, None, out)
         for s, _, _ in taken:
