@@ -97,11 +97,12 @@ class Attention:
 
     @classmethod
     def parameters(cls, spec, hidden):
-        params = {"q_proj.weight": ParamSpec((spec.q_width, hidden)),
-                  "o_proj.weight": ParamSpec((hidden, spec.out_width))}
+        # (in this order: a model of random weights draws them in the order of this table)
+        params = {"q_proj.weight": ParamSpec((spec.q_width, hidden))}
         if not spec.shared_kv:
             params["k_proj.weight"] = ParamSpec((spec.kv_width, hidden))
             params["v_proj.weight"] = ParamSpec((spec.v_width, hidden))
+        params["o_proj.weight"] = ParamSpec((hidden, spec.out_width))
         if spec.o_bias is not False:
             params["o_proj.bias"] = ParamSpec((hidden,), optional=spec.o_bias is not True)
         if spec.talking_heads:
