@@ -443,6 +443,27 @@ def test_window_attention_with_pooled_blocks_alone(shape, dtype):
                               max_rel=4e-2)
 
 
+@pytest.mark.parametrize("dim, heads, kv_heads", [(64, 8, 2), (128, 4, 1), (64, 3, 3)])
+def test_pooled_blocks_beside_the_matrix_core_kernel_whose_waves_take_whole_pages(dim, heads, kv_heads):
+    """A prompt of few blocks lets two waves share every page's keys; one of many blocks gives
+    a wave the whole page.  The second form is asked for here on a short prompt (the oracle
+    walks every pair of positions), with the pooled slice and the gate taken in at its end."""
+    mixer = window_spec(heads, kv_heads, dim, dim, 0.15, 40, 6, (1e4, dim // 2))
+    spec = one_layer(mixer)
+    params = params_for(spec, seed=17, gain=1.5)
+    model, session = session_for(spec, params, "bfloat16")
+    part = model.layers[0].mixer
+    assert part.pooled_aside
+    part.prefill_key_ways = lambda counts: 1
+    torch.manual_seed(3)
+    T = 200
+    x = torch.randn(T, HIDDEN).to(torch.bfloat16).float()
+    want, _ = plain_window(params, 0, mixer, x.double())
+    for cuts in ([T], [70, 130], [T - 3, 1, 1, 1]):
+        got, = in_cuts(session, [part], x, cuts)
+        assert_close_bf16(got, want, f"one wave a page, cuts {cuts}", rms_rel=2e-2, max_rel=4e-2)
+
+
 @pytest.mark.parametrize("dtype, dim", [("float32", 16), ("bfloat16", 64), ("bfloat16", 16)])
 @pytest.mark.parametrize("window, pool", [(5, 3), (64, 64), (65, 7), (100, 12), (6, 16)])
 def test_keys_that_stand_out_at_the_edges_of_window_and_blocks(window, pool, dtype, dim):
