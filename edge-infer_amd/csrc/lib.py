@@ -77,7 +77,8 @@ _SIGNATURES = {
     "norms": {
         "ei_stream_norm": [c_void_p, c_void_p, c_int, c_int, c_longlong, c_void_p, c_void_p,
                            c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_int, c_void_p, c_int,
-                           c_int, c_int, c_int, c_void_p],
+                           c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                           c_int, c_int, c_void_p],
         "ei_norm_mean": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_float,
                          c_void_p, c_int, c_int, c_void_p],
     },
@@ -1483,13 +1484,16 @@ def ssm_out(y_raw, proj, norm_w, eps, shape: SsmShape, parts, row_seq, out) -> N
 # ---------------------------------------------------------------------------
 def stream_norm(residual, delta, out, *, w_after=None, b_after=None, w_next=None, b_next=None,
                 eps: float, centred: bool, rows=None, write_residual: bool = True,
-                delta_bias=None) -> None:
+                delta_bias=None, conv=None) -> None:
     """One pass over the rows of the float32 stream `residual` [R, H].  With d the sum of
     delta's slices (+ delta_bias [H]): if `w_after` is given, d <- norm(d) * w_after + b_after
     (the norm on a sublayer's output); residual += d (stored back unless told not to); if
     `out` is given, out[i] = norm(residual[rows[i] if rows else i]) * w_next + b_next in out's
     type.  centred: norms with a mean (layer norms; the biases may be None), else RMS norms.
-    delta None: nothing is added."""
+    delta None: nothing is added.  conv = (weight [taps, H] float32, state, part, parts,
+    seq_in, seq_out) (a decode step only: row r is sequence r, widths that are multiples of
+    4): `out` receives h + conv(h) for the normed rows h, as `input_conv` gives it, and the
+    sequences' state moves on by the row."""
     lib = library("norms")
     total_rows, hidden = residual.shape
     n = total_rows if rows is None else rows.numel()
@@ -1510,13 +1514,28 @@ def stream_norm(residual, delta, out, *, w_after=None, b_after=None, w_next=None
 
     def f32(vector, name):
         return None if vector is None else _gpu(vector, name, torch.float32)
+    conv_args = (None, None, None, None, 0, 0, 0)
+    if conv is not None:
+        weight, state, part, parts, seq_in, seq_out = conv
+        taps = weight.shape[0]
+        if out is None or rows is not None or tuple(weight.shape) != (taps, hidden) or hidden % 4:
+            raise KernelError("stream_norm: the convolution needs normed rows that are the "
+                              "step's sequences and a width that is a multiple of 4")
+        if taps > 1 and (state is None or state.shape[1] != parts * (taps - 1) * hidden
+                         or seq_in.numel() < n or seq_out.numel() < n):
+            raise KernelError("stream_norm: the convolution's state does not fit")
+        conv_args = (_gpu(weight, "conv weight", torch.float32),
+                     None if taps == 1 else _gpu(state, "state", torch.float32),
+                     None if taps == 1 else _gpu(seq_in, "seq_in", torch.int32),
+                     None if taps == 1 else _gpu(seq_out, "seq_out", torch.int32), taps,
+                     int(part), int(parts))
     status = lib.ei_stream_norm(
         _gpu(residual, "residual", torch.float32), delta_ptr, delta_code, nsplit, stride,
         f32(delta_bias, "delta_bias"), None if rows is None else _gpu(rows, "rows", torch.int32),
         f32(w_after, "w_after"), f32(b_after, "b_after"), f32(w_next, "w_next"),
         f32(b_next, "b_next"), float(eps), int(bool(centred)),
         None if out is None else _gpu(out, "out"), F32 if out is None else _code(out, "out"), n,
-        hidden, int(write_residual), _stream())
+        hidden, int(write_residual), *conv_args, _stream())
     _check(lib, status, "stream_norm")
 
 

@@ -85,6 +85,22 @@ __global__ void stream_norm_kernel(float* __restrict__ residual, const TD* __res
 
 using ei::Vec4;
 
+// The short causal convolution of a step in which every sequence brings one token (a decode
+// step: row r is sequence r), taken in by the norm kernel that makes the convolution's input:
+// with h the normed row as it is stored, out = h + sum_j w[j] x_j, x_j the last taps - 1 inputs
+// of the sequence (its state, part `part` of row seq_in[r] of a table with two versions) and,
+// for the last tap, h itself; the state row seq_out[r] receives the inputs moved on by one.
+// w null: no convolution.  The sums are taken in the order of the kernel that convolves a
+// step's rows on its own, so a token gives the same values either way.
+struct ConvTail {
+  const float* w;          // [taps, H]
+  const float* state;      // rows of parts * (taps - 1) * H floats
+  float* state_out;        // (the same table)
+  const int32_t* seq_in;
+  const int32_t* seq_out;
+  int taps, part, parts;
+};
+
 // Four neighbouring elements of a row as the sum of its slices, in slice order; eight loads are
 // issued before the first sum, so that a row costs one trip to memory per eight slices.
 template <typename TD>
@@ -139,7 +155,8 @@ __global__ void stream_norm_vec_kernel(float* __restrict__ residual, const TD* _
                                        const float* __restrict__ b_after,
                                        const float* __restrict__ w_next,
                                        const float* __restrict__ b_next, float eps, int centred,
-                                       TO* __restrict__ out, int H, int write_residual) {
+                                       TO* __restrict__ out, int H, int write_residual,
+                                       ConvTail conv) {
   __shared__ float scratch[16];
   const int row = blockIdx.x;
   const int src = rows ? rows[row] : row;
@@ -216,6 +233,34 @@ __global__ void stream_norm_vec_kernel(float* __restrict__ residual, const TD* _
       if (b_next) Vec4<float>::load(b_next + qd * 4, b);
 #pragma unroll
       for (int i = 0; i < 4; ++i) z[i] = ((y[k][i] - mean) * inv) * w[i] + b[i];
+      if (conv.w) {
+        // the row as the next kernel would have read it, then its taps
+        float h[4], acc[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i] = h[i] = ei::to_f32<TO>(ei::from_f32<TO>(z[i]));
+        const int tail = conv.taps - 1;
+        const size_t row_floats = static_cast<size_t>(conv.parts) * tail * H;
+        const size_t at = static_cast<size_t>(conv.part) * tail * H + qd * 4;
+        const float* old = nullptr;
+        float* renewed = nullptr;
+        if (tail > 0) {
+          old = conv.state + static_cast<size_t>(conv.seq_in[row]) * row_floats + at;
+          renewed = conv.state_out + static_cast<size_t>(conv.seq_out[row]) * row_floats + at;
+        }
+        for (int j = 0; j < tail; ++j) {
+          float x[4], wj[4];
+          Vec4<float>::load(old + static_cast<size_t>(j) * H, x);
+          Vec4<float>::load(conv.w + static_cast<size_t>(j) * H + qd * 4, wj);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[i] += wj[i] * x[i];
+          if (j > 0) Vec4<float>::store(renewed + static_cast<size_t>(j - 1) * H, x);
+        }
+        float wl[4];
+        Vec4<float>::load(conv.w + static_cast<size_t>(tail) * H + qd * 4, wl);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) z[i] = acc[i] + wl[i] * h[i];
+        if (tail > 0) Vec4<float>::store(renewed + static_cast<size_t>(tail - 1) * H, h);
+      }
       Vec4<TO>::store(dst + qd * 4, z);
     }
   }
@@ -339,8 +384,16 @@ extern "C" int ei_stream_norm(float* residual, const void* delta, int delta_dtyp
                               const int32_t* rows, const float* w_after, const float* b_after,
                               const float* w_next, const float* b_next, float eps, int centred,
                               void* out, int out_dtype, int N, int H, int write_residual,
+                              const float* conv_w, float* conv_state, const int32_t* seq_in,
+                              const int32_t* seq_out, int taps, int part, int parts,
                               hipStream_t stream) {
   EI_REQUIRE(N > 0 && H > 0, "stream_norm: sizes must be positive");
+  const ConvTail conv{conv_w, conv_state, conv_state, seq_in, seq_out, taps, part, parts};
+  EI_REQUIRE(!conv_w || (out && !rows && taps >= 1 && taps <= 64 && parts >= 1 && part >= 0 &&
+                         part < parts && (taps == 1 || (conv_state && seq_in && seq_out)) &&
+                         H % 4 == 0 && (!delta || split_stride % 4 == 0) && H <= 16384),
+             "stream_norm: the convolution of a decode step needs rows that are sequences, its "
+             "state and a width that is a multiple of 4");
   EI_REQUIRE(residual, "stream_norm: null pointer");
   EI_REQUIRE(!delta || nsplit >= 1, "stream_norm: nsplit must be at least 1");
   EI_REQUIRE(delta || !w_after, "stream_norm: a norm on a sublayer's output needs that output");
@@ -358,7 +411,7 @@ extern "C" int ei_stream_norm(float* residual, const void* delta, int delta_dtyp
 #define EI_SN_VEC(TD, TO, C)                                                                   \
   stream_norm_vec_kernel<TD, TO, C><<<N, vthreads, 0, stream>>>(                               \
       residual, static_cast<const TD*>(delta), nsplit, ss, delta_bias, rows, w_after, b_after, \
-      w_next, b_next, eps, centred, static_cast<TO*>(out), H, write_residual)
+      w_next, b_next, eps, centred, static_cast<TO*>(out), H, write_residual, conv)
 #define EI_SN(TD, TO)                                                                          \
   do {                                                                                         \
     if (chunks == 1) EI_SN_VEC(TD, TO, 1);                                                     \

@@ -339,6 +339,7 @@ class SandwichBlock:
                          for norm in (self.norm1b, self.norm2) if norm is not None)
         self.fused_own = (self.norm2 is not None and hasattr(self.norm1b, "norm_add_then")
                           and type(self.norm1b) is type(self.norm2))
+        self.hidden = hidden
         self.taps = int(getattr(layer_spec, "input_conv", 0))
         self.conv1 = self.conv2 = None
         if self.taps:
@@ -346,6 +347,19 @@ class SandwichBlock:
             self.conv1 = params["conv1.weight"].to(device=device, dtype=torch.float32).t().contiguous()
             if self.ffn is not None:
                 self.conv2 = params["conv2.weight"].to(device=device, dtype=torch.float32).t().contiguous()
+
+    def _conv_in_norm(self, ctx, entry, part, norm):
+        """What the norm kernel needs to take the convolution of sublayer `part` in itself, or
+        None where it cannot: in a step whose sequences bring one token each, a row's taps are
+        its own sequence's state, so the norm that makes the row can add them."""
+        widths = getattr(norm, "conv_widths", 0)
+        if not (self.taps and ctx.decode and widths and self.hidden % widths == 0):
+            return None
+        state = seq_in = seq_out = None
+        if self.taps > 1:
+            state = ctx.cache.state((entry.own_id, self.CONV_STATE))
+            seq_in, seq_out = ctx.meta.seq_state_in, ctx.meta.seq_state_out
+        return (self.conv1 if part == 0 else self.conv2, state, part, 2, seq_in, seq_out)
 
     def _convolved(self, ctx, h, entry, part):
         """h + conv(h) for sublayer `part` (0: the mixer, 1: the feed-forward)."""
@@ -365,8 +379,10 @@ class SandwichBlock:
         if pending is not None:
             raise ValueError("sandwich: a delta of the block before is still pending; this "
                              "arrangement follows only blocks that add everything themselves")
-        h = self.norm1.add_norm(ctx, residual, None, "block.h", write_residual=False)
-        if self.taps:
+        conv = self._conv_in_norm(ctx, entry, 0, self.norm1)
+        h = self.norm1.add_norm(ctx, residual, None, "block.h", write_residual=False,
+                                **({} if conv is None else {"conv": conv}))
+        if self.taps and conv is None:
             h = self._convolved(ctx, h, entry, 0)
         # a sublayer that can leave its last product's bias to the norm kernel behind it does
         a, a_bias = (self.mixer.forward(ctx, h, entry, bias_later=True)
@@ -377,17 +393,23 @@ class SandwichBlock:
             self.norm1b.norm_add(ctx, residual, a, bias=a_bias)
             ctx.release(a)
             return None
+        conv = None
         if self.fused:
             h2 = ctx.buffer("block.h", tuple(residual.shape))
             lib.norm_add_norm(residual, a, self.norm1b.weight, self.norm2.weight, self.norm2.eps, h2,
                               bias=a_bias)
-        elif self.fused_own:
-            h2 = self.norm1b.norm_add_then(ctx, residual, a, self.norm2, "block.h", bias=a_bias)
         else:
-            self.norm1b.norm_add(ctx, residual, a, bias=a_bias)
-            h2 = self.norm2.add_norm(ctx, residual, None, "block.h", write_residual=False)
+            conv = self._conv_in_norm(ctx, entry, 1, self.norm2)
+            more = {} if conv is None else {"conv": conv}
+            if self.fused_own:
+                h2 = self.norm1b.norm_add_then(ctx, residual, a, self.norm2, "block.h", bias=a_bias,
+                                               **more)
+            else:
+                self.norm1b.norm_add(ctx, residual, a, bias=a_bias)
+                h2 = self.norm2.add_norm(ctx, residual, None, "block.h", write_residual=False,
+                                         **more)
         ctx.release(a)
-        if self.taps:
+        if self.taps and conv is None:
             h2 = self._convolved(ctx, h2, entry, 1)
         f, f_bias = (self.ffn.forward(ctx, h2, bias_later=True)
                      if getattr(self.ffn, "bias_later", False)

@@ -78,13 +78,16 @@ class LayerNorm:
         self.weight = (self.weight * vector).contiguous()
         self.bias = (self.bias * vector).contiguous()
 
-    def add_norm(self, ctx, residual, delta, out_name, rows=None, write_residual=True):
+    conv_widths = 4      # `conv` of the two methods below is taken for widths that are multiples
+
+    def add_norm(self, ctx, residual, delta, out_name, rows=None, write_residual=True, conv=None):
         """residual += delta (all splits); returns layernorm(residual)[rows] in the step's
-        storage type."""
+        storage type.  `conv` (a decode step only; see `lib.stream_norm`): the rows returned
+        are h + conv(h) for the normed rows h."""
         n = residual.shape[0] if rows is None else rows.numel()
         out = ctx.buffer(out_name, (n, self.width))
         lib.stream_norm(residual, delta, out, w_next=self.weight, b_next=self.bias, eps=self.eps,
-                        centred=True, rows=rows, write_residual=write_residual)
+                        centred=True, rows=rows, write_residual=write_residual, conv=conv)
         return out
 
     def norm_add(self, ctx, residual, delta, cast_name=None, bias=None):
@@ -96,11 +99,12 @@ class LayerNorm:
                         eps=self.eps, centred=True, delta_bias=bias)
         return None
 
-    def norm_add_then(self, ctx, residual, delta, following, out_name, bias=None):
+    def norm_add_then(self, ctx, residual, delta, following, out_name, bias=None, conv=None):
         """residual += layernorm(delta (+ bias)), and then the rows of `following`, a norm of
-        this kind before the next sublayer, in one pass: returns following(residual)."""
+        this kind before the next sublayer, in one pass: returns following(residual) (with
+        `conv`, a decode step only: those rows with their convolution added)."""
         out = ctx.buffer(out_name, tuple(residual.shape))
         lib.stream_norm(residual, delta, out, w_after=self.weight, b_after=self.bias,
                         w_next=following.weight, b_next=following.bias, eps=self.eps,
-                        centred=True, delta_bias=bias)
+                        centred=True, delta_bias=bias, conv=conv)
         return out

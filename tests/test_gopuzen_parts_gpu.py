@@ -570,3 +570,42 @@ def test_a_layer_that_reads_another_layers_keys(dtype):
             else:
                 assert_close_bf16(got, want, f"{what}, cuts {cuts[:3]}", rms_rel=2e-2, max_rel=4e-2)
     session.cache.check()
+
+
+@pytest.mark.parametrize("taps, width", [(3, 48), (1, 64), (4, 2048)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_a_decode_steps_convolution_inside_the_norm_kernel(taps, width, dtype):
+    """A step whose sequences bring one token each: the norm kernel adds the taps itself.  The
+    rows it writes and the state it leaves are, bit for bit, those of the norm followed by the
+    convolution kernel, token after token, for three sequences side by side."""
+    from edge_infer_amd.csrc import lib
+    g = torch.Generator().manual_seed(taps + width)
+    w = exact((width, taps), g, 0.5).t().contiguous().to(DEV)
+    weight, bias = exact((width,), g).to(DEV), exact((width,), g).to(DEV)
+    seqs, floats = 3, 2 * max(taps - 1, 0) * width
+    states = [torch.zeros(2 * (seqs + 1), max(floats, 1), device=DEV) for _ in range(2)]
+
+    def i32(values):
+        return torch.tensor(values, dtype=torch.int32, device=DEV)
+    version = 0
+    for token in range(7):
+        residual = exact((seqs, width), g, 2.0).to(DEV)
+        seq_in = i32([version * (seqs + 1) + s for s in range(seqs)])
+        seq_out = i32([(1 - version) * (seqs + 1) + s for s in range(seqs)])
+        # apart: the norm, then the convolution of the step's rows
+        h = torch.empty(seqs, width, device=DEV, dtype=dtype)
+        lib.stream_norm(residual, None, h, w_next=weight, b_next=bias, eps=EPS, centred=True,
+                        write_residual=False)
+        apart = torch.empty_like(h)
+        lib.input_conv(h, w, states[0] if taps > 1 else None, 1, 2, i32([token] * seqs),
+                       i32(list(range(seqs))), seq_in, seq_out, i32([token] * seqs), i32([1] * seqs),
+                       i32(list(range(seqs))), apart)
+        # in one kernel
+        fused = torch.empty_like(h)
+        lib.stream_norm(residual, None, fused, w_next=weight, b_next=bias, eps=EPS, centred=True,
+                        write_residual=False,
+                        conv=(w, states[1] if taps > 1 else None, 1, 2, seq_in, seq_out))
+        assert torch.equal(fused, apart), f"token {token}"
+        if taps > 1:
+            assert torch.equal(states[0], states[1]), f"state after token {token}"
+        version ^= 1
