@@ -72,8 +72,14 @@ attn_generic_kernel(const T* __restrict__ q, const T* __restrict__ k_pages,
   const float slope = (slopes && row_valid) ? slopes[head] : 0.f;
   const int chunk_r = (chunk > 0 && row_valid) ? pos_r / chunk : 0;
 
+  // (the pooled entries alone, and the item's last row sees none: nothing to meet)
+  bool idle = false;
+  if (pool_only && seq >= 0 && npos > 0) {
+    const int before = row_pos[row0 + npos - 1] - window + 1;
+    idle = before < pool;
+  }
   // query rows, pre-scaled
-  for (int idx = t; idx < kRows * DQ; idx += kThreads) {
+  for (int idx = t; idx < kRows * DQ && !idle; idx += kThreads) {
     const int rr = idx / DQ, d = idx % DQ;
     const int ppi = rr / Gb, hhi = hb * Gb + rr % Gb;
     float v = 0.f;
@@ -168,7 +174,7 @@ attn_generic_kernel(const T* __restrict__ q, const T* __restrict__ k_pages,
       }
   };
 
-  if (seq >= 0 && npos > 0) {
+  if (seq >= 0 && npos > 0 && !idle) {
     const int hi_key = row_pos[row0 + npos - 1];
     int lo_key = window > 0 ? max(0, row_pos[row0] - window + 1) : 0;
     if (chunk > 0) lo_key = max(lo_key, row_pos[row0] / chunk * chunk);
@@ -393,13 +399,17 @@ __global__ void pool_store_kernel(const T* __restrict__ k_pages, const T* __rest
                                   const int32_t* __restrict__ page_table,
                                   const int32_t* __restrict__ pool_table, int table_width,
                                   T* __restrict__ pool_k, T* __restrict__ pool_v, int N, int nkv,
-                                  int D, int DV, int P, int pieces) {
+                                  int D, int DV, int P, int pieces,
+                                  const int32_t* __restrict__ row_list) {
   // a wave a (row, kv head, piece of 64 elements of [key | value]); eight positions' loads
   // are issued before the first is added
   const int wave = (blockIdx.x * blockDim.x + threadIdx.x) / EI_WAVE;
   const int lane = threadIdx.x % EI_WAVE;
   if (wave >= N * nkv * pieces) return;
-  const int piece = wave % pieces, g = wave / pieces % nkv, row = wave / pieces / nkv;
+  const int piece = wave % pieces, g = wave / pieces % nkv;
+  // (row_list: the rows that end a block, as the host has worked them out; -1: none)
+  const int row = row_list ? row_list[wave / pieces / nkv] : wave / pieces / nkv;
+  if (row < 0) return;
   const int seq = row_seq[row];
   if (seq < 0) return;
   const int pos = row_pos[row];
@@ -438,29 +448,34 @@ __global__ void pool_store_kernel(const T* __restrict__ k_pages, const T* __rest
 
 // k_pages [pages, nkv, 64, D], v_pages [pages, nkv, 64, DV] hold the tokens; pool_k, pool_v the
 // same shapes for the pooled entries, found through pool_table as tokens are through page_table.
+// row_list (or null): n_listed rows to look at instead of all N (a prompt step's rows that end a
+// block, known to the host; entries of -1 are skipped).
 extern "C" int ei_pool_store(const void* k_pages, const void* v_pages, int dtype,
                              const int32_t* row_pos, const int32_t* row_seq,
                              const int32_t* page_table, const int32_t* pool_table, int table_width,
                              void* pool_k, void* pool_v, int N, int nkv, int D, int DV, int P,
-                             hipStream_t stream) {
+                             const int32_t* row_list, int n_listed, hipStream_t stream) {
   EI_REQUIRE(k_pages && v_pages && row_pos && row_seq && page_table && pool_table && pool_k && pool_v,
              "pool_store: null pointer");
   EI_REQUIRE(N > 0 && nkv > 0 && D > 0 && DV > 0 && P >= 1 && table_width > 0,
              "pool_store: sizes must be positive");
   const int pieces = (D + DV + EI_WAVE - 1) / EI_WAVE;
-  const size_t waves = static_cast<size_t>(N) * nkv * pieces;
+  EI_REQUIRE(!row_list || n_listed > 0, "pool_store: an empty list of rows");
+  // N rows, or only the listed ones among them
+  const size_t waves = static_cast<size_t>(row_list ? n_listed : N) * nkv * pieces;
+  if (row_list) N = n_listed;
   EI_REQUIRE(waves * EI_WAVE / 256 < 0x7fffffffULL, "pool_store: too many rows for one launch");
   const unsigned blocks = static_cast<unsigned>((waves * EI_WAVE + 255) / 256);
   if (dtype == EI_F32)
     pool_store_kernel<float><<<blocks, 256, 0, stream>>>(
         static_cast<const float*>(k_pages), static_cast<const float*>(v_pages), row_pos, row_seq,
         page_table, pool_table, table_width, static_cast<float*>(pool_k),
-        static_cast<float*>(pool_v), N, nkv, D, DV, P, pieces);
+        static_cast<float*>(pool_v), N, nkv, D, DV, P, pieces, row_list);
   else if (dtype == EI_BF16)
     pool_store_kernel<bf16_t><<<blocks, 256, 0, stream>>>(
         static_cast<const bf16_t*>(k_pages), static_cast<const bf16_t*>(v_pages), row_pos, row_seq,
         page_table, pool_table, table_width, static_cast<bf16_t*>(pool_k),
-        static_cast<bf16_t*>(pool_v), N, nkv, D, DV, P, pieces);
+        static_cast<bf16_t*>(pool_v), N, nkv, D, DV, P, pieces, row_list);
   else
     EI_REQUIRE(false, "pool_store: unknown dtype");
   EI_LAUNCH_CHECK();

@@ -128,7 +128,8 @@ _SIGNATURES = {
                          c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float,
                          c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p],
         "ei_pool_store": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
-                          c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+                          c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int,
+                          c_void_p],
     },
     "attention_wide": {
         "ei_attn_wide_supported": [c_int, c_int, c_int],
@@ -676,9 +677,10 @@ def attention(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items, row_
 
 
 def pool_store(k_pages, v_pages, row_pos, row_seq, page_table, pool_table, pool_k, pool_v, n_rows,
-               pool) -> None:
+               pool, row_list=None) -> None:
     """For every row whose position ends a block of `pool` positions: the means of the block's
-    cached keys and values (all kv heads) into entry position // pool of the pooled cache."""
+    cached keys and values (all kv heads) into entry position // pool of the pooled cache.
+    row_list (int32, optional): the rows to look at instead of all `n_rows` (-1: skipped)."""
     lib = library("attention_generic")
     n_kv_heads, head_dim, value_dim = k_pages.shape[1], k_pages.shape[3], v_pages.shape[3]
     if tuple(pool_k.shape[1:]) != tuple(k_pages.shape[1:]) or \
@@ -693,7 +695,9 @@ def pool_store(k_pages, v_pages, row_pos, row_seq, page_table, pool_table, pool_
         _gpu(row_pos, "row_pos", torch.int32), _gpu(row_seq, "row_seq", torch.int32),
         _gpu(page_table, "page_table", torch.int32), _gpu(pool_table, "pool_table", torch.int32),
         page_table.shape[-1], _gpu(pool_k, "pool_k"), _gpu(pool_v, "pool_v"), n_rows, n_kv_heads,
-        head_dim, value_dim, int(pool), _stream())
+        head_dim, value_dim, int(pool),
+        None if row_list is None else _gpu(row_list, "row_list", torch.int32),
+        0 if row_list is None else row_list.numel(), _stream())
     _check(lib, status, "pool_store")
 
 

@@ -363,7 +363,7 @@ class Attention:
     def plan_key(self):
         """Attention parts with equal keys plan the same sections."""
         return ("attention", self.positions_per_item(), self.group, self.spec.n_kv_heads, self.wide,
-                self.pooled_aside)
+                self.pooled_aside, self.spec.pool)
 
     def _items_section(self, key_ways: int = 1):
         return f"attention.items{self.positions_per_item(key_ways)}"
@@ -399,6 +399,12 @@ class Attention:
             name = f"attention.items{self._aside_size()}"
             if name not in sections:
                 sections[name] = self._prompt_items(plan, self._aside_size())
+        if self.spec.pool is not None:
+            # the rows of this step that end a block of `pool` positions (-1: there is none)
+            pool = self.spec.pool
+            rows = [seq.row0 + k for seq in plan.seqs
+                    for k in range((-(seq.start + 1)) % pool, seq.count, pool)]
+            sections[f"attention.pool_rows{pool}"] = np.asarray(rows or [-1], dtype=np.int32)
         return sections
 
     @staticmethod
@@ -520,7 +526,9 @@ class Attention:
                 pool_group, pool_k, pool_v = ctx.cache.kv((entry.own_id, self.POOL))
                 pool_table = meta.page_table(pool_group)
                 lib.pool_store(k_pages, v_pages, meta.row_pos, meta.row_seq, page_table,
-                               pool_table, pool_k, pool_v, n, spec.pool)
+                               pool_table, pool_k, pool_v, n, spec.pool,
+                               row_list=None if ctx.decode else
+                               meta.section(f"attention.pool_rows{spec.pool}"))
                 pooled = dict(pool=spec.pool, pool_k=pool_k, pool_v=pool_v, pool_table=pool_table)
                 if self.pooled_aside:
                     # every row's sums over the pooled blocks it sees, for the matrix-core
